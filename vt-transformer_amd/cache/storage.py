@@ -77,10 +77,13 @@ class CacheStorage:
         needs: List[Optional[CacheNeed]] = []
         state_needs: List[Optional[StateNeed]] = []
         for i, e in enumerate(schedule):
-            mixer = model.layers[e.layer].mixer
+            block = model.layers[e.layer]
+            mixer = block.mixer
             need = mixer.cache_need() if hasattr(mixer, "cache_need") else None
             needs.append(need)
-            state_needs.append(mixer.state_need() if hasattr(mixer, "state_need") else None)
+            # (a block that keeps state of its own between steps declares it together with its mixer's)
+            holder = block if hasattr(block, "state_need") else mixer
+            state_needs.append(holder.state_need() if hasattr(holder, "state_need") else None)
             if e.cache_from is not None:
                 src = needs[e.cache_from]
                 if need is None or src is None or not need.same_layout(src):

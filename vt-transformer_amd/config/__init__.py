@@ -3,10 +3,13 @@ from .registry import architectures, config_from_dict, load_config, register_arc
 from .qwen2 import Qwen2Config
 from .lisunex import LisunexConfig
 from .gabelorn import GabelornConfig
+from .kigalix import KigalixConfig
 
 register_architecture(Qwen2Config.architecture, Qwen2Config)
 register_architecture(LisunexConfig.architecture, LisunexConfig)
 register_architecture(GabelornConfig.architecture, GabelornConfig)
+register_architecture(KigalixConfig.architecture, KigalixConfig)
 
 __all__ = ["ConfigError", "LayerSpec", "ModelConfig", "ModelSpec", "PartSpec", "ScheduleEntry",
-           "architectures", "config_from_dict", "load_config", "register_architecture", "Qwen2Config", "LisunexConfig", "GabelornConfig"]
+           "architectures", "config_from_dict", "load_config", "register_architecture", "Qwen2Config", "LisunexConfig", "GabelornConfig",
+           "KigalixConfig"]

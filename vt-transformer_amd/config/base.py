@@ -82,9 +82,17 @@ class ModelSpec:
     # a tensor [rows, hidden_size] of vectors that schedule entries add to the stream before they run
     # (``ScheduleEntry.offset_row``): {"name": tensor name, "rows": number of rows}
     stream_offsets: Optional[Dict[str, Any]] = None
+    # 0: one residual stream [tokens, width].  S >= 1: S copies of it, [tokens, S, width], which all start as the
+    # embedding's output and are added up in front of the final norm; the layers' blocks are then of a kind that
+    # reads and writes several streams ("hyper")
+    streams: int = 0
 
     def validate(self) -> None:
         n = len(self.layers)
+        if self.streams < 0:
+            raise ConfigError(f"{self.streams} residual streams")
+        if self.streams and self.stream_offsets:
+            raise ConfigError("stream offsets are added to a single residual stream only")
         for i, e in enumerate(self.schedule):
             if e.offset_row is not None:
                 rows = int(self.stream_offsets["rows"]) if self.stream_offsets else 0
@@ -119,6 +127,10 @@ class ModelConfig:
 
     def to_spec(self) -> ModelSpec:
         raise NotImplementedError
+
+    def take_tensor_shapes(self, shapes: Dict[str, Any]) -> None:
+        """Called with the shapes of a checkpoint's tensors by name before the model is built from it: a
+        configuration fills in here the sizes that only the tensors give and its config.json does not."""
 
     def save(self, folder: str) -> None:
         os.makedirs(folder, exist_ok=True)

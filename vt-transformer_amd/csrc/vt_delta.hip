@@ -14,7 +14,15 @@
 //                         add their shares up by rotations within the row.  Tokens are taken in tiles of 16 through
 //                         LDS; every token is computed by the same instructions in the same order whatever the
 //                         tile, so a result does not depend on how the request was cut into steps.
-//   vt_gated_rmsnorm:     out = o / rms(o) * w * silu(gate), per (token, head).
+//   vt_gated_rmsnorm:     out = o / rms(o) * w * silu(gate) (or sigmoid(gate)), per (token, head); w shared by the heads
+//                         or one per head.
+//
+// The generalized delta rule beside it: a decay per key channel instead of one per head, and what is taken out of
+// the state lies along the unit key, scaled per channel:
+//     S <- diag(w) S - (a * u)(u^T S) + k v^T,  u = k / sqrt(|k|^2 + eps);   o = S^T r      (both terms read the old S)
+// with w = exp(-c * sigmoid(z)) from decay logits z and a = sigmoid(removal logits), all in float32.
+//   vt_lowrank_tanh:      z[t][j] = bias[j] + sum_l W2[j][l] tanh(x[t][l]): the decay logits from a low-rank projection.
+//   vt_general_delta:     the recurrence, in vt_delta_rule's arrangement (a row of 16 lanes per state column).
 #include "vt_common.h"
 #include <math.h>
 
@@ -345,36 +353,235 @@ extern "C" int vt_delta_rule(const void* qkv, int dtype, const void* ba, int ba_
 }
 
 // ---------------------------------------------------------------------------
-// out[t][h][:] = o[t][h][:] / sqrt(mean(o^2) + eps) * w[:] * silu(gate[t][h][:]); gate[t * ldg + h * Dv + j]
+// out[t][h][:] = o[t][h][:] / sqrt(mean(o^2) + eps) * w[h * w_stride + :] * act(gate[t][h][:]); gate[t * ldg + h * Dv + j];
+// act: silu (gate_kind 0) or sigmoid (1); w_stride 0: one weight vector for all heads, Dv: one per head
 template <typename TG, typename TO>
 __global__ __launch_bounds__(64) void gated_rmsnorm_kernel(const float* __restrict__ o, const float* __restrict__ w,
                                                            const TG* __restrict__ gate, long long ldg, TO* __restrict__ out,
-                                                           int H, int Dv, float eps) {
+                                                           int H, int Dv, float eps, int w_stride, int gate_kind) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const float* row = o + ((size_t)t * H + h) * Dv;
+    const float* wh = w + (size_t)h * w_stride;
     float ss = 0.f;
     for (int j = lane; j < Dv; j += 64) ss = fmaf(row[j], row[j], ss);
     ss = wave_sum(ss);
     const float rinv = 1.0f / sqrtf(ss / (float)Dv + eps);
     for (int j = lane; j < Dv; j += 64) {
         const float z = load_f32<TG>(gate, (size_t)t * ldg + (size_t)h * Dv + j);
-        store_f32<TO>(out, ((size_t)t * H + h) * Dv + j, row[j] * rinv * w[j] * silu_f(z));
+        const float g = gate_kind ? 1.0f / (1.0f + expf(-z)) : silu_f(z);
+        store_f32<TO>(out, ((size_t)t * H + h) * Dv + j, row[j] * rinv * wh[j] * g);
     }
 }
 
 extern "C" int vt_gated_rmsnorm(const float* o, const float* w, const void* gate, int gate_dtype, long long ldg, void* out,
-                                int out_dtype, int n, int H, int Dv, float eps, hipStream_t stream) {
+                                int out_dtype, int n, int H, int Dv, float eps, int w_per_head, int gate_kind,
+                                hipStream_t stream) {
     VT_REQUIRE(n >= 0 && H > 0 && Dv > 0 && H <= 65535, "vt_gated_rmsnorm: bad sizes");
     VT_REQUIRE(ldg >= (long long)H * Dv, "vt_gated_rmsnorm: gate rows are too short");
+    VT_REQUIRE(gate_kind == 0 || gate_kind == 1, "vt_gated_rmsnorm: gate kind %d (0: silu, 1: sigmoid)", gate_kind);
     if (n == 0) return 0;
     const dim3 grid(n, H);
+    const int ws = w_per_head ? Dv : 0;
     if (gate_dtype == VT_F32 && out_dtype == VT_F32)
-        gated_rmsnorm_kernel<float, float><<<grid, 64, 0, stream>>>(o, w, (const float*)gate, ldg, (float*)out, H, Dv, eps);
+        gated_rmsnorm_kernel<float, float><<<grid, 64, 0, stream>>>(o, w, (const float*)gate, ldg, (float*)out, H, Dv, eps, ws, gate_kind);
     else if (gate_dtype == VT_F32 && out_dtype == VT_BF16)
-        gated_rmsnorm_kernel<float, bf16_t><<<grid, 64, 0, stream>>>(o, w, (const float*)gate, ldg, (bf16_t*)out, H, Dv, eps);
+        gated_rmsnorm_kernel<float, bf16_t><<<grid, 64, 0, stream>>>(o, w, (const float*)gate, ldg, (bf16_t*)out, H, Dv, eps, ws, gate_kind);
     else if (gate_dtype == VT_BF16 && out_dtype == VT_BF16)
-        gated_rmsnorm_kernel<bf16_t, bf16_t><<<grid, 64, 0, stream>>>(o, w, (const bf16_t*)gate, ldg, (bf16_t*)out, H, Dv, eps);
+        gated_rmsnorm_kernel<bf16_t, bf16_t><<<grid, 64, 0, stream>>>(o, w, (const bf16_t*)gate, ldg, (bf16_t*)out, H, Dv, eps, ws, gate_kind);
     else return vt_fail("vt_gated_rmsnorm: dtypes %d -> %d are not handled", gate_dtype, out_dtype);
     VT_CHECK_LAUNCH("vt_gated_rmsnorm");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// z[t][j] = bias[j] + sum_l W2[j][l] * tanh(x[t * ldx + l]), l = 0, 1, .. in that order, float32
+template <typename TI, typename TW>
+__global__ __launch_bounds__(256) void lowrank_tanh_kernel(const TI* __restrict__ x, long long ldx, const TW* __restrict__ w2,
+                                                           const float* __restrict__ bias, float* __restrict__ z, int L, int M) {
+    extern __shared__ float th[];
+    const int t = blockIdx.x;
+    for (int l = threadIdx.x; l < L; l += 256) th[l] = tanhf(load_f32<TI>(x, (size_t)t * ldx + l));
+    __syncthreads();
+    const int j = blockIdx.y * 256 + threadIdx.x;
+    if (j >= M) return;
+    float acc = bias ? bias[j] : 0.f;
+    for (int l = 0; l < L; ++l) acc = fmaf(load_f32<TW>(w2, (size_t)j * L + l), th[l], acc);
+    z[(size_t)t * M + j] = acc;
+}
+
+extern "C" int vt_lowrank_tanh(const void* x, int x_dtype, long long ldx, const void* w2, int w_dtype, const float* bias,
+                               float* z, int n, int L, int M, hipStream_t stream) {
+    VT_REQUIRE(n >= 0 && L > 0 && L <= 8192 && M > 0 && ldx >= L, "vt_lowrank_tanh: bad sizes n=%d L=%d M=%d", n, L, M);
+    VT_REQUIRE(M <= 65535 * 256, "vt_lowrank_tanh: too many outputs");
+    if (n == 0) return 0;
+    const dim3 grid(n, (M + 255) / 256);
+    const size_t lds = (size_t)L * sizeof(float);
+    if (x_dtype == VT_F32 && w_dtype == VT_F32)
+        lowrank_tanh_kernel<float, float><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const float*)w2, bias, z, L, M);
+    else if (x_dtype == VT_F32 && w_dtype == VT_BF16)
+        lowrank_tanh_kernel<float, bf16_t><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const bf16_t*)w2, bias, z, L, M);
+    else if (x_dtype == VT_BF16 && w_dtype == VT_BF16)
+        lowrank_tanh_kernel<bf16_t, bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w2, bias, z, L, M);
+    else return vt_fail("vt_lowrank_tanh: dtypes %d / %d are not handled", x_dtype, w_dtype);
+    VT_CHECK_LAUNCH("vt_lowrank_tanh");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+struct GeneralDeltaArgs {
+    const void* x;          // [n][ldx]: per head D read-out elements from column r_col, D keys from k_col, Dv values
+                            // from v_col, D removal logits from a_col (heads one behind the other)
+    const float* z;         // [n][H * D] decay logits, float32
+    const float* a_bias;    // [H * D] or null: added to the removal logits
+    float* state;           // slot s: state + s * slot_stride, [H][Dv][D]
+    const int* entry_start;
+    const int* slots;
+    float* o;               // [n][H][Dv]
+    long long ldx, slot_stride;
+    int r_col, k_col, v_col, a_col;
+    int H, D, Dv;
+    float decay_scale, key_eps;
+};
+
+// vt_delta_rule's arrangement: the block's 256 threads are 16 rows of lanes for the recurrence (a row per value
+// column, lane r holding the state elements d = 16 i + r) and TILE tokens x 16 lanes for a tile's inputs, which are
+// asked for before the recurrence over the tile in front starts.  Per token and column:
+//     p = u . S;   S_d <- w_d S_d - (a_d u_d) p + k_d v;   o = r . S
+// the same instructions in the same order whatever the tile, so nothing depends on how a request was cut.
+template <typename TI, int DS, int TILE>
+__global__ __launch_bounds__(256) void general_delta_kernel(GeneralDeltaArgs a) {
+    constexpr int DP = 16 * DS;
+    __shared__ float rs[TILE][DP];      // read-out vectors
+    __shared__ float ks[TILE][DP];      // keys as they come
+    __shared__ float us[TILE][DP];      // unit keys
+    __shared__ float bs[TILE][DP];      // removal rate times unit key
+    __shared__ float ws[TILE][DP];      // decays
+    __shared__ float vs[TILE][DELTA_GROUPS];
+
+    const int e = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * DELTA_GROUPS;
+    const int tid = threadIdx.x;
+    const int r = tid & 15, cl = tid >> 4;
+    const int D = a.D, Dv = a.Dv, H = a.H;
+    const int start = a.entry_start[e], end = a.entry_start[e + 1];
+    float* S_head = a.state + (size_t)a.slots[e] * a.slot_stride + (size_t)h * Dv * D;
+    const TI* x = (const TI*)a.x;
+    const int col = col0 + cl;
+
+    float S[DS];
+#pragma unroll
+    for (int i = 0; i < DS; ++i) {
+        const int d = 16 * i + r;
+        S[i] = (col < Dv && d < D) ? S_head[(size_t)col * D + d] : 0.f;
+    }
+    float ab[DS];
+#pragma unroll
+    for (int i = 0; i < DS; ++i) {
+        const int d = 16 * i + r;
+        ab[i] = (a.a_bias && d < D) ? a.a_bias[(size_t)h * D + d] : 0.f;
+    }
+
+    float in_r[DS], in_k[DS], in_a[DS], in_z[DS], in_v = 0.f;
+    auto fetch = [&](int t0) {
+        const int t = t0 + cl;
+        const bool ok = cl < TILE && t < end;
+        const size_t row = (size_t)(ok ? t : start) * a.ldx;
+        const size_t zrow = (size_t)(ok ? t : start) * H * D + (size_t)h * D;
+#pragma unroll
+        for (int i = 0; i < DS; ++i) {
+            const int d = 16 * i + r;
+            const bool in = ok && d < D;
+            in_r[i] = in ? load_f32<TI>(x, row + a.r_col + (size_t)h * D + d) : 0.f;
+            in_k[i] = in ? load_f32<TI>(x, row + a.k_col + (size_t)h * D + d) : 0.f;
+            in_a[i] = in ? load_f32<TI>(x, row + a.a_col + (size_t)h * D + d) : 0.f;
+            in_z[i] = in ? a.z[zrow + d] : 0.f;
+        }
+        const int j = col0 + r;
+        in_v = (ok && j < Dv) ? load_f32<TI>(x, row + a.v_col + (size_t)h * Dv + j) : 0.f;
+    };
+    fetch(start);
+    for (int t0 = start; t0 < end; t0 += TILE) {
+        const int nt = min(TILE, end - t0);
+        __syncthreads();        // the tile before has been read
+        if (cl < TILE) {
+            float sk = 0.f;
+#pragma unroll
+            for (int i = 0; i < DS; ++i) sk = fmaf(in_k[i], in_k[i], sk);
+            sk = row16_sum(sk);
+            const float rk = 1.0f / sqrtf(sk + a.key_eps);
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                const int d = 16 * i + r;
+                const float u = in_k[i] * rk;
+                const float rate = 1.0f / (1.0f + expf(-(in_a[i] + ab[i])));
+                rs[cl][d] = in_r[i];
+                ks[cl][d] = in_k[i];
+                us[cl][d] = u;
+                bs[cl][d] = rate * u;
+                ws[cl][d] = expf(-a.decay_scale / (1.0f + expf(-in_z[i])));
+            }
+            vs[cl][r] = in_v;
+        }
+        __syncthreads();
+        if (t0 + TILE < end) fetch(t0 + TILE);      // on its way while this tile is worked through
+        auto token = [&](int tt) {
+            float p = 0.f;
+#pragma unroll
+            for (int i = 0; i < DS; ++i) p = fmaf(us[tt][16 * i + r], S[i], p);
+            p = row16_sum(p);
+            const float v = vs[tt][cl];
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                const int d = 16 * i + r;
+                S[i] = fmaf(ws[tt][d], S[i], fmaf(-bs[tt][d], p, ks[tt][d] * v));
+                acc = fmaf(rs[tt][d], S[i], acc);
+            }
+            acc = row16_sum(acc);
+            if (r == 0 && col < Dv) a.o[((size_t)(t0 + tt) * H + h) * Dv + col] = acc;
+        };
+        if (nt == TILE) {
+#pragma unroll
+            for (int tt = 0; tt < TILE; ++tt) token(tt);
+        } else {
+            for (int tt = 0; tt < nt; ++tt) token(tt);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < DS; ++i) {
+        const int d = 16 * i + r;
+        if (col < Dv && d < D) S_head[(size_t)col * D + d] = S[i];
+    }
+}
+
+extern "C" int vt_general_delta(const void* x, int dtype, long long ldx, int r_col, int k_col, int v_col, int a_col,
+                                const float* z, const float* a_bias, float* state, long long slot_stride,
+                                const int* entry_start, const int* slots, float* o, int n_entries, int H, int D, int Dv,
+                                float decay_scale, float key_eps, hipStream_t stream) {
+    VT_REQUIRE(n_entries >= 0 && H > 0 && H <= 65535, "vt_general_delta: bad heads %d", H);
+    VT_REQUIRE(D > 0 && D <= 256 && Dv > 0, "vt_general_delta: head sizes %d/%d (keys up to 256)", D, Dv);
+    VT_REQUIRE(slot_stride >= (long long)H * D * Dv, "vt_general_delta: state slots are too short");
+    VT_REQUIRE(min(min(r_col, k_col), min(v_col, a_col)) >= 0 && ldx >= max(max(r_col, k_col), a_col) + (long long)H * D &&
+               ldx >= v_col + (long long)H * Dv, "vt_general_delta: rows are too short for their columns");
+    VT_REQUIRE(decay_scale > 0.f && key_eps >= 0.f, "vt_general_delta: bad constants");
+    if (n_entries == 0) return 0;
+    GeneralDeltaArgs a;
+    a.x = x; a.z = z; a.a_bias = a_bias; a.state = state; a.entry_start = entry_start; a.slots = slots; a.o = o;
+    a.ldx = ldx; a.slot_stride = slot_stride; a.r_col = r_col; a.k_col = k_col; a.v_col = v_col; a.a_col = a_col;
+    a.H = H; a.D = D; a.Dv = Dv; a.decay_scale = decay_scale; a.key_eps = key_eps;
+    const int share = (D + 15) / 16;
+    const dim3 grid(n_entries, H, (Dv + DELTA_GROUPS - 1) / DELTA_GROUPS);
+#define VT_GDELTA(TI)                                                                              \
+    do {                                                                                           \
+        if (share <= 1) general_delta_kernel<TI, 1, 16><<<grid, 256, 0, stream>>>(a);              \
+        else if (share <= 2) general_delta_kernel<TI, 2, 16><<<grid, 256, 0, stream>>>(a);         \
+        else if (share <= 4) general_delta_kernel<TI, 4, 16><<<grid, 256, 0, stream>>>(a);         \
+        else if (share <= 8) general_delta_kernel<TI, 8, 16><<<grid, 256, 0, stream>>>(a);         \
+        else general_delta_kernel<TI, 16, 8><<<grid, 256, 0, stream>>>(a);                         \
+    } while (0)
+    if (dtype == VT_F32) VT_GDELTA(float);
+    else if (dtype == VT_BF16) VT_GDELTA(bf16_t);
+    else return vt_fail("vt_general_delta: unknown dtype %d", dtype);
+#undef VT_GDELTA
+    VT_CHECK_LAUNCH("vt_general_delta");
     return 0;
 }

@@ -348,28 +348,29 @@ extern "C" int vt_silu_mul(const void* gu, int in_dtype, void* out, int out_dtyp
 
 // ---------------------------------------------------------------------------
 // A gated unit with bounds: g = min(gu[t, i], limit), u = clamp(gu[t, inter + i], -limit, limit),
-// out[t, i] = g * sigmoid(alpha * g) * (u + shift).  limit <= 0: no bounds.  (alpha 1, shift 0 and no bounds is
-// vt_silu_mul.)  A thread takes four columns where the width is a multiple of 4.
+// out[t, i] = g * sigmoid(alpha * g * (1 + cubic * g^2)) * (u + shift).  limit <= 0: no bounds.  (alpha 1, shift 0,
+// cubic 0 and no bounds is vt_silu_mul; alpha 2 sqrt(2 / pi) and cubic 0.044715 is the tanh form of GELU.)  A thread takes four columns where the width is a multiple of 4.
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ float bounded_gate(float g, float u, float alpha, float limit, float shift) {
+__device__ __forceinline__ float bounded_gate(float g, float u, float alpha, float limit, float shift, float cubic) {
     if (limit > 0.f) {
         g = fminf(g, limit);
         u = fminf(fmaxf(u, -limit), limit);
     }
-    return g / (1.f + expf(-alpha * g)) * (u + shift);
+    const float z = cubic != 0.f ? alpha * g * fmaf(cubic * g, g, 1.f) : alpha * g;
+    return g / (1.f + expf(-z)) * (u + shift);
 }
 template <typename TI, typename TO>
 __global__ void gated_act_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter, float alpha, float limit,
-                                 float shift) {
+                                 float shift, float cubic) {
     int t = blockIdx.y;
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= inter) return;
     const TI* row = gu + (size_t)t * 2 * inter;
-    store_f32<TO>(out + (size_t)t * inter, i, bounded_gate(load_f32<TI>(row, i), load_f32<TI>(row, (size_t)inter + i), alpha, limit, shift));
+    store_f32<TO>(out + (size_t)t * inter, i, bounded_gate(load_f32<TI>(row, i), load_f32<TI>(row, (size_t)inter + i), alpha, limit, shift, cubic));
 }
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void gated_act_vec_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter,
-                                                           int n, float alpha, float limit, float shift) {
+                                                           int n, float alpha, float limit, float shift, float cubic) {
     const int qpr = inter >> 2;
     const long long total = (long long)qpr * n;
     for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long long)gridDim.x * 256) {
@@ -378,26 +379,27 @@ __global__ __launch_bounds__(256) void gated_act_vec_kernel(const TI* __restrict
         const TI* row = gu + (size_t)t * 2 * inter;
         const float4 g = load4(row + i), u = load4(row + inter + i);
         store4(out + (size_t)t * inter + i,
-               make_float4(bounded_gate(g.x, u.x, alpha, limit, shift), bounded_gate(g.y, u.y, alpha, limit, shift),
-                           bounded_gate(g.z, u.z, alpha, limit, shift), bounded_gate(g.w, u.w, alpha, limit, shift)));
+               make_float4(bounded_gate(g.x, u.x, alpha, limit, shift, cubic), bounded_gate(g.y, u.y, alpha, limit, shift, cubic),
+                           bounded_gate(g.z, u.z, alpha, limit, shift, cubic), bounded_gate(g.w, u.w, alpha, limit, shift, cubic)));
     }
 }
 // 16-bit in and out, widths that are a multiple of 8: silu_mul_bf16x8_kernel's arrangement (a thread takes eight
 // columns in four rows, eight 16-byte loads asked for before any is used, marked non-temporal)
 // (the division as one reciprocal instruction, 1 ulp, far below the 16-bit rounding of the result)
-__device__ __forceinline__ float bounded_gate_fast(float g, float u, float alpha, float limit, float shift) {
+__device__ __forceinline__ float bounded_gate_fast(float g, float u, float alpha, float limit, float shift, float cubic) {
     if (limit > 0.f) {
         g = fminf(g, limit);
         u = fminf(fmaxf(u, -limit), limit);
     }
-    return g * __builtin_amdgcn_rcpf(1.f + __expf(-alpha * g)) * (u + shift);
+    const float z = cubic != 0.f ? alpha * g * fmaf(cubic * g, g, 1.f) : alpha * g;
+    return g * __builtin_amdgcn_rcpf(1.f + __expf(-z)) * (u + shift);
 }
-__device__ __forceinline__ unsigned bounded_gate_pair(unsigned g, unsigned u, float alpha, float limit, float shift) {
-    return vt_pack2(bounded_gate_fast(lowp_lo(g), lowp_lo(u), alpha, limit, shift),
-                    bounded_gate_fast(lowp_hi(g), lowp_hi(u), alpha, limit, shift));
+__device__ __forceinline__ unsigned bounded_gate_pair(unsigned g, unsigned u, float alpha, float limit, float shift, float cubic) {
+    return vt_pack2(bounded_gate_fast(lowp_lo(g), lowp_lo(u), alpha, limit, shift, cubic),
+                    bounded_gate_fast(lowp_hi(g), lowp_hi(u), alpha, limit, shift, cubic));
 }
 __global__ __launch_bounds__(256) void gated_act_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
-                                                              int inter, int n, float alpha, float limit, float shift) {
+                                                              int inter, int n, float alpha, float limit, float shift, float cubic) {
     typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
     const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
     if (c >= inter) return;
@@ -415,38 +417,38 @@ __global__ __launch_bounds__(256) void gated_act_bf16x8_kernel(const bf16_t* __r
     for (int k = 0; k < 4; ++k) {
         if (t0 + k < n) {
             u32x4_t o;
-            o.x = bounded_gate_pair(g[k].x, u[k].x, alpha, limit, shift); o.y = bounded_gate_pair(g[k].y, u[k].y, alpha, limit, shift);
-            o.z = bounded_gate_pair(g[k].z, u[k].z, alpha, limit, shift); o.w = bounded_gate_pair(g[k].w, u[k].w, alpha, limit, shift);
+            o.x = bounded_gate_pair(g[k].x, u[k].x, alpha, limit, shift, cubic); o.y = bounded_gate_pair(g[k].y, u[k].y, alpha, limit, shift, cubic);
+            o.z = bounded_gate_pair(g[k].z, u[k].z, alpha, limit, shift, cubic); o.w = bounded_gate_pair(g[k].w, u[k].w, alpha, limit, shift, cubic);
             *(u32x4_t*)(out + (size_t)(t0 + k) * inter + c) = o;
         }
     }
 }
 template <typename TI, typename TO>
-static void launch_gated_act(const void* gu, void* out, int n, int inter, float alpha, float limit, float shift,
+static void launch_gated_act(const void* gu, void* out, int n, int inter, float alpha, float limit, float shift, float cubic,
                              hipStream_t stream) {
     if constexpr (sizeof(TI) == 2 && sizeof(TO) == 2) {
         if (inter % 8 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)out & 15)) {
             const dim3 grid((inter / 8 + 255) / 256, (n + 3) / 4);
-            gated_act_bf16x8_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, n, alpha, limit, shift);
+            gated_act_bf16x8_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, n, alpha, limit, shift, cubic);
             return;
         }
     }
     if (inter % 4 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)out & 15)) {
         long long blocks = ((long long)(inter / 4) * n + 255) / 256;
         if (blocks > 16384) blocks = 16384;
-        gated_act_vec_kernel<TI, TO><<<(unsigned)blocks, 256, 0, stream>>>((const TI*)gu, (TO*)out, inter, n, alpha, limit, shift);
+        gated_act_vec_kernel<TI, TO><<<(unsigned)blocks, 256, 0, stream>>>((const TI*)gu, (TO*)out, inter, n, alpha, limit, shift, cubic);
     } else {
-        gated_act_kernel<TI, TO><<<dim3((inter + 255) / 256, n), 256, 0, stream>>>((const TI*)gu, (TO*)out, inter, alpha, limit, shift);
+        gated_act_kernel<TI, TO><<<dim3((inter + 255) / 256, n), 256, 0, stream>>>((const TI*)gu, (TO*)out, inter, alpha, limit, shift, cubic);
     }
 }
 extern "C" int vt_gated_act(const void* gu, int in_dtype, void* out, int out_dtype, int n, int inter, float alpha,
-                            float limit, float shift, hipStream_t stream) {
+                            float limit, float shift, float cubic, hipStream_t stream) {
     VT_REQUIRE(n >= 0 && inter > 0, "vt_gated_act: bad sizes n=%d inter=%d", n, inter);
     if (n == 0) return 0;
     VT_REQUIRE(n <= 65535, "vt_gated_act: more than 65535 rows (%d)", n);
-    if (in_dtype == VT_F32 && out_dtype == VT_F32) launch_gated_act<float, float>(gu, out, n, inter, alpha, limit, shift, stream);
-    else if (in_dtype == VT_F32 && out_dtype == VT_BF16) launch_gated_act<float, bf16_t>(gu, out, n, inter, alpha, limit, shift, stream);
-    else if (in_dtype == VT_BF16 && out_dtype == VT_BF16) launch_gated_act<bf16_t, bf16_t>(gu, out, n, inter, alpha, limit, shift, stream);
+    if (in_dtype == VT_F32 && out_dtype == VT_F32) launch_gated_act<float, float>(gu, out, n, inter, alpha, limit, shift, cubic, stream);
+    else if (in_dtype == VT_F32 && out_dtype == VT_BF16) launch_gated_act<float, bf16_t>(gu, out, n, inter, alpha, limit, shift, cubic, stream);
+    else if (in_dtype == VT_BF16 && out_dtype == VT_BF16) launch_gated_act<bf16_t, bf16_t>(gu, out, n, inter, alpha, limit, shift, cubic, stream);
     else return vt_fail("vt_gated_act: unknown dtypes %d -> %d", in_dtype, out_dtype);
     VT_CHECK_LAUNCH("vt_gated_act");
     return 0;

@@ -41,11 +41,12 @@ int vt_linear_bf16_fused(const void* h, const float* gain, float eps, const void
 int vt_gated_linear_bf16(const void* x, const void* wp, void* y, int out_dtype, int N, int I, int K,
                          const float* gain, float eps, hipStream_t stream);
 // the same with biases (bias[0..I) the gate's, bias[I..2I) the up projection's, or null) and a gate of the form
-// g = min(g, limit), u = clamp(u, -limit, limit) (limit 0: no bounds), g * sigmoid(alpha * g) * (u + shift); the norm
+// g = min(g, limit), u = clamp(u, -limit, limit) (limit 0: no bounds), g * sigmoid(alpha * g * (1 + cubic * g^2)) *
+// (u + shift); the norm
 // in front applied here (gain, eps) or prepared by the product in front (ssq_in, n_ssq, eps), or neither
 int vt_gated_linear_bf16_form(const void* x, const void* wp, const float* bias, void* y, int out_dtype, int N, int I,
                               int K, const float* gain, float eps, const float* ssq_in, int n_ssq, float alpha,
-                              float limit, float shift, hipStream_t stream);
+                              float limit, float shift, float cubic, hipStream_t stream);
 
 // An RMSNorm handed from the product in front of it (which adds to the residual stream and writes, beside it, the
 // stream times the norm's gains in bfloat16 and its blocks' shares of the rows' sums of squares) to the product

@@ -138,17 +138,20 @@ __device__ __forceinline__ bf16x8_t load_x(const bf16_t* row, int k, int K) {
 // since it is the same for a whole row.  The shares are added in a fixed order: the result does not depend on
 // which block finished first.  Rows of ssq are SSQ_STRIDE(N) floats apart.
 // The form of the gated product's gate, with g and u the two matrices' sums (and their biases, if any):
-//     g <- min(g, limit), u <- clamp(u, -limit, limit)   (limit 0: no bounds);   g * sigmoid(alpha * g) * (u + shift).
-// alpha 1, limit 0, shift 0 is SiLU gating, to the bit what it was before the form had parameters.
+//     g <- min(g, limit), u <- clamp(u, -limit, limit)   (limit 0: no bounds);
+//     g * sigmoid(alpha * g * (1 + cubic * g^2)) * (u + shift).
+// alpha 1, limit 0, shift 0, cubic 0 is SiLU gating, to the bit what it was before the form had parameters;
+// alpha 2 sqrt(2 / pi), cubic 0.044715 is the tanh form of GELU, since (1 + tanh z) / 2 = sigmoid(2 z).
 struct GateForm {
-    float alpha, limit, shift;
+    float alpha, limit, shift, cubic;
 };
 __device__ __forceinline__ float gate_form(float g, float u, const GateForm& f) {
     if (f.limit > 0.f) {
         g = fminf(g, f.limit);
         u = fminf(fmaxf(u, -f.limit), f.limit);
     }
-    return g / (1.f + expf(-f.alpha * g)) * (u + f.shift);
+    const float z = f.cubic != 0.f ? f.alpha * g * fmaf(f.cubic * g, g, 1.f) : f.alpha * g;
+    return g / (1.f + expf(-z)) * (u + f.shift);
 }
 struct NormLink {
     bf16_t* xn_out;            // producer: [N][Mout], or null
@@ -994,7 +997,7 @@ extern "C" long long vt_linear_bf16_workspace(int N, int M, int K, int gated) {
 
 // gain != null: x is the fp32 residual stream and the RMSNorm (gain, eps) is part of the product (up to 16 tokens);
 // resid != null: the result is added to it (up to 64 tokens).
-static const NormLink NO_LINK = {nullptr, nullptr, nullptr, nullptr, 0, 0.f, {1.f, 0.f, 0.f}};
+static const NormLink NO_LINK = {nullptr, nullptr, nullptr, nullptr, 0, 0.f, {1.f, 0.f, 0.f, 0.f}};
 
 // shares of the rows' sums of squares that a producing product of this shape writes (0: it cannot produce)
 extern "C" int vt_linear_bf16_link_shares(int N, int M, int K) {
@@ -1194,7 +1197,7 @@ extern "C" int vt_linear_bf16_link(const void* x, const void* wp, const float* b
                                    void* xn_out, const float* gain_next, float* ssq_out, hipStream_t stream) {
     VT_REQUIRE(N >= 0 && M > 0 && K > 0, "vt_linear_bf16_link: bad sizes N=%d M=%d K=%d", N, M, K);
     VT_REQUIRE(ssq_in || xn_out, "vt_linear_bf16_link: neither end of a norm: use vt_linear_bf16");
-    const NormLink link = {(bf16_t*)xn_out, gain_next, ssq_out, ssq_in, n_ssq, eps_in, {1.f, 0.f, 0.f}};
+    const NormLink link = {(bf16_t*)xn_out, gain_next, ssq_out, ssq_in, n_ssq, eps_in, {1.f, 0.f, 0.f, 0.f}};
     return linear_bf16<false, float>(x, (const bf16_t*)wp, bias, y, workspace, N, M, K, nullptr, 0.f, resid, stream, link);
 }
 
@@ -1203,7 +1206,7 @@ extern "C" int vt_gated_linear_bf16_link(const void* x, const void* wp, void* y,
                                          const float* ssq_in, int n_ssq, float eps_in, hipStream_t stream) {
     VT_REQUIRE(N >= 0 && I > 0 && K > 0, "vt_gated_linear_bf16_link: bad sizes N=%d I=%d K=%d", N, I, K);
     VT_REQUIRE(ssq_in, "vt_gated_linear_bf16_link: no sums of squares: use vt_gated_linear_bf16");
-    const NormLink link = {nullptr, nullptr, nullptr, ssq_in, n_ssq, eps_in, {1.f, 0.f, 0.f}};
+    const NormLink link = {nullptr, nullptr, nullptr, ssq_in, n_ssq, eps_in, {1.f, 0.f, 0.f, 0.f}};
     if (out_dtype == VT_F32) return linear_bf16<true, float>(x, (const bf16_t*)wp, nullptr, (float*)y, nullptr, N, I, K, nullptr, 0.f, nullptr, stream, link);
     if (out_dtype == VT_BF16) return linear_bf16<true, bf16_t>(x, (const bf16_t*)wp, nullptr, (bf16_t*)y, nullptr, N, I, K, nullptr, 0.f, nullptr, stream, link);
     return vt_fail("vt_gated_linear_bf16_link: unknown out dtype %d", out_dtype);
@@ -1215,11 +1218,11 @@ extern "C" int vt_gated_linear_bf16_link(const void* x, const void* wp, void* y,
 // front has prepared (n_ssq, eps as above).
 extern "C" int vt_gated_linear_bf16_form(const void* x, const void* wp, const float* bias, void* y, int out_dtype, int N,
                                          int I, int K, const float* gain, float eps, const float* ssq_in, int n_ssq,
-                                         float alpha, float limit, float shift, hipStream_t stream) {
+                                         float alpha, float limit, float shift, float cubic, hipStream_t stream) {
     VT_REQUIRE(N >= 0 && I > 0 && K > 0, "vt_gated_linear_bf16_form: bad sizes N=%d I=%d K=%d", N, I, K);
     VT_REQUIRE(!(gain && ssq_in), "vt_gated_linear_bf16_form: a norm in front is applied here or was prepared, not both");
     VT_REQUIRE(alpha > 0.f && limit >= 0.f, "vt_gated_linear_bf16_form: bad gate (alpha %g, limit %g)", alpha, limit);
-    const NormLink link = {nullptr, nullptr, nullptr, ssq_in, ssq_in ? n_ssq : 0, ssq_in ? eps : 0.f, {alpha, limit, shift}};
+    const NormLink link = {nullptr, nullptr, nullptr, ssq_in, ssq_in ? n_ssq : 0, ssq_in ? eps : 0.f, {alpha, limit, shift, cubic}};
     const float* g = ssq_in ? nullptr : gain;
     if (out_dtype == VT_F32) return linear_bf16<true, float>(x, (const bf16_t*)wp, bias, (float*)y, nullptr, N, I, K, g, eps, nullptr, stream, link);
     if (out_dtype == VT_BF16) return linear_bf16<true, bf16_t>(x, (const bf16_t*)wp, bias, (bf16_t*)y, nullptr, N, I, K, g, eps, nullptr, stream, link);

@@ -11,6 +11,7 @@ from ..models.model import DecoderModel
 from ..parts.base import Runtime
 from ..weights.loader import check_tensors, load_model_weights
 from ..weights.random_init import random_tensor
+from ..weights.safetensors_io import WeightStore
 from .step import ModelRunner
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float16": torch.float16, "fp16": torch.float16,
@@ -39,7 +40,15 @@ def load_model(folder: str, dtype, device: Optional[torch.device] = None, keep_r
                page_size: Optional[int] = None) -> DecoderModel:
     """config.json chooses the architecture; model.safetensors (or its shards) gives the tensors.  With `page_size`
     the model's parts are asked whether they take it before any tensor is read."""
-    model = build_model(load_config(folder), dtype, device, keep_row_major)
+    config = load_config(folder)
+    if type(config).take_tensor_shapes is not ModelConfig.take_tensor_shapes:
+        # a design whose config.json leaves sizes to the tensors' shapes
+        store = WeightStore(folder)
+        try:
+            config.take_tensor_shapes({n: tuple(store.info(n)[1]) for n in store.names()})
+        finally:
+            store.close()
+    model = build_model(config, dtype, device, keep_row_major)
     if page_size is not None:
         check_page_size(model, page_size)
     load_model_weights(model, folder)

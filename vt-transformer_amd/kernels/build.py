@@ -30,11 +30,13 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-shared",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 # libraries that every model needs; attention for the 16-bit types is built per head size
-BASE_LIBS = ["vt_elementwise", "vt_gemm_f32", "vt_gemm_bf16", "vt_attn_f32", "vt_attn_masked", "vt_delta", "vt_latent", "vt_sampling"]
+BASE_LIBS = ["vt_elementwise", "vt_gemm_f32", "vt_gemm_bf16", "vt_attn_f32", "vt_attn_masked", "vt_delta", "vt_latent", "vt_streams",
+             "vt_moe", "vt_sampling"]
 DEFAULT_HEAD_DIMS = list(range(16, 257, 16))
 # The libraries that handle 16-bit values are built once for bfloat16 and once for float16 (-DVT_LOWP_F16: the same
 # sources with the other conversion and the other matrix instruction); the float16 build's name ends in _f16.
-HALF_LIBS = ("vt_elementwise", "vt_gemm_bf16", "vt_attn_bf16", "vt_attn_masked", "vt_attn_masked_mfma", "vt_delta", "vt_latent")
+HALF_LIBS = ("vt_elementwise", "vt_gemm_bf16", "vt_attn_bf16", "vt_attn_masked", "vt_attn_masked_mfma", "vt_delta", "vt_latent",
+             "vt_streams", "vt_moe")
 # the matrix-core kernel of the masked attention is built per (key size, value size) of a head
 DEFAULT_MASKED_DIMS = [(64, 64), (128, 128), (64, 96), (48, 80), (32, 48), (16, 16), (64, 32), (64, 16), (48, 32), (256, 192)]
 

@@ -158,9 +158,10 @@ def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def gated_act(gu: torch.Tensor, out: torch.Tensor, alpha: float = 1.0, limit: float = 0.0, shift: float = 0.0) -> torch.Tensor:
-    """gu [n, 2 I] (gate columns, then up columns) -> out [n, I] = g sigmoid(alpha g) (u + shift) with g = min(gate,
-    limit) and u = clamp(up, -limit, limit); limit 0: no bounds."""
+def gated_act(gu: torch.Tensor, out: torch.Tensor, alpha: float = 1.0, limit: float = 0.0, shift: float = 0.0,
+              cubic: float = 0.0) -> torch.Tensor:
+    """gu [n, 2 I] (gate columns, then up columns) -> out [n, I] = g sigmoid(alpha g (1 + cubic g^2)) (u + shift) with
+    g = min(gate, limit) and u = clamp(up, -limit, limit); limit 0: no bounds."""
     n, two_i = gu.shape
     _chk(gu, "gated_act.gu")
     _chk(out, "gated_act.out", None, (n, two_i // 2))
@@ -169,7 +170,7 @@ def gated_act(gu: torch.Tensor, out: torch.Tensor, alpha: float = 1.0, limit: fl
     if out.dtype == torch.float32 and gu.dtype != torch.float32:
         raise KernelError("gated_act: float32 results need float32 inputs")
     _run(load_lib("vt_elementwise", half=_half(gu, out)), "vt_gated_act", _ptr(gu), _i(_code(gu)), _ptr(out), _i(_code(out)),
-         _i(n), _i(two_i // 2), _f(alpha), _f(limit), _f(shift), _stream())
+         _i(n), _i(two_i // 2), _f(alpha), _f(limit), _f(shift), _f(cubic), _stream())
     return out
 
 
@@ -499,8 +500,8 @@ def gated_linear_bf16(x: torch.Tensor, w_gate_up, out: torch.Tensor, norm_gain: 
 
 def gated_linear_bf16_form(x: torch.Tensor, w: PackedMatrix, bias: Optional[torch.Tensor], out: torch.Tensor,
                            alpha: float, limit: float, shift: float, norm_gain: Optional[torch.Tensor] = None,
-                           norm_eps: float = 0.0, ssq_in: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out = gate(x Wg^T + bias[:I], x Wu^T + bias[I:]) with gate(g, u) = g' sigmoid(alpha g') (u' + shift),
+                           norm_eps: float = 0.0, ssq_in: Optional[torch.Tensor] = None, cubic: float = 0.0) -> torch.Tensor:
+    """out = gate(x Wg^T + bias[:I], x Wu^T + bias[I:]) with gate(g, u) = g' sigmoid(alpha g' (1 + cubic g'^2)) (u' + shift),
     g' = min(g, limit), u' = clamp(u, -limit, limit) (limit 0: no bounds); w: two packed halves.  x: 16-bit tokens;
     or with norm_gain the float32 residual stream whose RMSNorm is what gets multiplied (up to 16 rows); or with
     ssq_in a norm that the product in front has prepared (gated_linear_bf16_link's x and ssq_in, eps in norm_eps)."""
@@ -530,7 +531,7 @@ def gated_linear_bf16_form(x: torch.Tensor, w: PackedMatrix, bias: Optional[torc
         raise KernelError(f"gated_linear_bf16_form: gate with alpha {alpha} and limit {limit}")
     _run(load_lib("vt_gemm_bf16", half=_half(w.data, x, out)), "vt_gated_linear_bf16_form", _ptr(x), _ptr(w.data), _ptr(bias),
          _ptr(out), _i(_code(out)), _i(n), _i(w.rows), _i(k), _ptr(norm_gain), _f(norm_eps), _ptr(ssq_in), _i(n_ssq),
-         _f(alpha), _f(limit), _f(shift), _stream())
+         _f(alpha), _f(limit), _f(shift), _f(cubic), _stream())
     return out
 
 
@@ -1103,18 +1104,201 @@ def delta_rule(qkv: torch.Tensor, ba: torch.Tensor, ba_column: int, a_log: torch
 
 
 def gated_rmsnorm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, gate_column: int, out: torch.Tensor,
-                  n_heads: int, value_dim: int, eps: float) -> torch.Tensor:
-    """out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * weight * silu(gate[t, gate_column + h * Dv ...]), per head."""
+                  n_heads: int, value_dim: int, eps: float, gate_kind: str = "silu") -> torch.Tensor:
+    """out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * weight * act(gate[t, gate_column + h * Dv ...]), per head;
+    weight [Dv] (shared by the heads) or [H * Dv] (one per head); gate_kind "silu" or "sigmoid"."""
     n = o.shape[0]
     _chk(o, "gated_rmsnorm.o", torch.float32, (n, n_heads * value_dim))
-    _chk(weight, "gated_rmsnorm.weight", torch.float32, (value_dim,))
+    _chk(weight, "gated_rmsnorm.weight", torch.float32)
+    if tuple(weight.shape) not in ((value_dim,), (n_heads * value_dim,)):
+        raise KernelError(f"gated_rmsnorm.weight: shape {tuple(weight.shape)}, expected ({value_dim},) or ({n_heads * value_dim},)")
+    per_head = tuple(weight.shape) == (n_heads * value_dim,) and n_heads > 1
+    if gate_kind not in ("silu", "sigmoid"):
+        raise KernelError(f"gated_rmsnorm: gate kind {gate_kind!r} ('silu' and 'sigmoid' are known)")
     _chk(gate, "gated_rmsnorm.gate")
     _chk(out, "gated_rmsnorm.out", None, (n, n_heads * value_dim))
     if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + n_heads * value_dim:
         raise KernelError(f"gated_rmsnorm.gate: shape {tuple(gate.shape)} has no {n_heads * value_dim} columns from {gate_column}")
     gptr = ctypes.c_void_p(gate.data_ptr() + gate_column * gate.element_size())
     _run(load_lib("vt_delta", half=_half(gate, out)), "vt_gated_rmsnorm", _ptr(o), _ptr(weight), gptr, _i(_code(gate)),
-         ctypes.c_longlong(gate.stride(0)), _ptr(out), _i(_code(out)), _i(n), _i(n_heads), _i(value_dim), _f(eps), _stream())
+         ctypes.c_longlong(gate.stride(0)), _ptr(out), _i(_code(out)), _i(n), _i(n_heads), _i(value_dim), _f(eps),
+         _i(1 if per_head else 0), _i(1 if gate_kind == "sigmoid" else 0), _stream())
+    return out
+
+
+def lowrank_tanh(x: torch.Tensor, x_column: int, w2: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+    """out[t, j] = bias[j] + sum_l w2[j, l] * tanh(x[t, x_column + l]): float32 sums in the order of l, float32 results.
+    x: a 2-d tensor whose rows are the tokens'; w2 [M, L] in float32 or the 16-bit type."""
+    n = x.shape[0]
+    m, low = w2.shape
+    _chk(x, "lowrank_tanh.x")
+    _chk(w2, "lowrank_tanh.w2")
+    if x.dim() != 2 or x_column < 0 or x.shape[1] < x_column + low:
+        raise KernelError(f"lowrank_tanh.x: shape {tuple(x.shape)} has no {low} columns from {x_column}")
+    if x.dtype != torch.float32 and w2.dtype != x.dtype:
+        raise KernelError(f"lowrank_tanh: inputs of {x.dtype} beside a matrix of {w2.dtype}")
+    if bias is not None:
+        _chk(bias, "lowrank_tanh.bias", torch.float32, (m,))
+    _chk(out, "lowrank_tanh.out", torch.float32, (n, m))
+    xptr = ctypes.c_void_p(x.data_ptr() + x_column * x.element_size())
+    _run(load_lib("vt_delta", half=_half(x, w2)), "vt_lowrank_tanh", xptr, _i(_code(x)), ctypes.c_longlong(x.stride(0)),
+         _ptr(w2), _i(_code(w2)), _ptr(bias), _ptr(out), _i(n), _i(low), _i(m), _stream())
+    return out
+
+
+def general_delta(x: torch.Tensor, r_column: int, k_column: int, v_column: int, a_column: int, decay_logits: torch.Tensor,
+                  a_bias: Optional[torch.Tensor], state: torch.Tensor, entry_start: torch.Tensor, slots: torch.Tensor,
+                  out: torch.Tensor, n_heads: int, key_dim: int, value_dim: int, decay_scale: float, key_eps: float) -> torch.Tensor:
+    """The generalized delta rule over the tokens of every entry, from and into state[slot] ([H, Dv, D] float32):
+    S <- diag(w) S - (a u)(u^T S) + k v^T, o = S^T r, with u = k / sqrt(|k|^2 + key_eps), w = exp(-decay_scale *
+    sigmoid(decay_logits)) and a = sigmoid(removal logits + a_bias).  x: a 2-d tensor whose rows are the tokens', with
+    H heads of D read-out elements from r_column, of D keys from k_column, of Dv values from v_column and of D removal
+    logits from a_column; decay_logits [n, H * D] float32; out [n, H * Dv] float32."""
+    n = x.shape[0]
+    hd = n_heads * key_dim
+    _chk(x, "general_delta.x")
+    if x.dim() != 2 or min(r_column, k_column, v_column, a_column) < 0 or \
+            x.shape[1] < max(max(r_column, k_column, a_column) + hd, v_column + n_heads * value_dim):
+        raise KernelError(f"general_delta.x: shape {tuple(x.shape)} does not hold its columns")
+    _chk(decay_logits, "general_delta.decay_logits", torch.float32, (n, hd))
+    if a_bias is not None:
+        _chk(a_bias, "general_delta.a_bias", torch.float32, (hd,))
+    _chk(out, "general_delta.out", torch.float32, (n, n_heads * value_dim))
+    _chk(entry_start, "general_delta.entry_start", torch.int32)
+    _chk(slots, "general_delta.slots", torch.int32)
+    if not 1 <= key_dim <= DELTA_MAX_KEY_DIM:
+        raise KernelError(f"general_delta: keys of {key_dim} (up to {DELTA_MAX_KEY_DIM})")
+    sp, ss = _state_rows(state, "general_delta", n_heads * key_dim * value_dim)
+    _run(load_lib("vt_delta", half=_half(x)), "vt_general_delta", _ptr(x), _i(_code(x)), ctypes.c_longlong(x.stride(0)),
+         _i(r_column), _i(k_column), _i(v_column), _i(a_column), _ptr(decay_logits), _ptr(a_bias), sp, ss, _ptr(entry_start),
+         _ptr(slots), _ptr(out), _i(entry_start.numel() - 1), _i(n_heads), _i(key_dim), _i(value_dim), _f(decay_scale),
+         _f(key_eps), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+# several residual streams and the token shift (vt_streams.hip)
+STREAMS_MAX = 8
+
+
+def streams_fill(h: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """x [n, S, W] float32: every stream of a token starts as h[token] (h [n, W] float32)."""
+    n, s, w = x.shape
+    _chk(h, "streams_fill.h", torch.float32, (n, w))
+    _chk(x, "streams_fill.x", torch.float32)
+    _run(load_lib("vt_streams"), "vt_streams_fill", _ptr(h), _ptr(x), _i(n), _i(s), _i(w), _stream())
+    return x
+
+
+def streams_read(x: torch.Tensor, w_in: torch.Tensor, gain: torch.Tensor, out: torch.Tensor, eps: float,
+                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[r] = RMSNorm(sum_s w_in[s] x[t, s]; gain, eps) with t = rows[r] (or r); x [n, S, W] float32, out [R, W] in
+    float32 or a 16-bit type."""
+    n, s, w = x.shape
+    _chk(x, "streams_read.x", torch.float32)
+    _chk(w_in, "streams_read.w_in", torch.float32, (s,))
+    _chk(gain, "streams_read.gain", torch.float32, (w,))
+    if not 1 <= s <= STREAMS_MAX:
+        raise KernelError(f"streams_read: {s} streams (1 to {STREAMS_MAX})")
+    r = n
+    if rows is not None:
+        _chk(rows, "streams_read.rows", torch.int32)
+        r = rows.numel()
+    _chk(out, "streams_read.out", None, (r, w))
+    _run(load_lib("vt_streams", half=_half(out)), "vt_streams_read", _ptr(x), _ptr(w_in), _ptr(gain), _ptr(rows), _ptr(out),
+         _i(_code(out)), _i(r), _i(s), _i(w), _f(eps), _stream())
+    return out
+
+
+def streams_write(x: torch.Tensor, mix: torch.Tensor, w_out: torch.Tensor, y: torch.Tensor,
+                  gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x[t, to] <- sum_s mix[s, to] x[t, s] + w_out[to] * y[t] * sigmoid(gate[t]) (no gate: without the factor), all
+    streams at once from the old ones; x [n, S, W] float32 in place, y and gate [n, W]."""
+    n, s, w = x.shape
+    _chk(x, "streams_write.x", torch.float32)
+    _chk(mix, "streams_write.mix", torch.float32, (s, s))
+    _chk(w_out, "streams_write.w_out", torch.float32, (s,))
+    _chk(y, "streams_write.y", None, (n, w))
+    if gate is not None:
+        _chk(gate, "streams_write.gate", None, (n, w))
+    if not 1 <= s <= STREAMS_MAX:
+        raise KernelError(f"streams_write: {s} streams (1 to {STREAMS_MAX})")
+    _run(load_lib("vt_streams", half=_half(y, gate)), "vt_streams_write", _ptr(x), _ptr(mix), _ptr(w_out), _ptr(y),
+         _i(_code(y)), _ptr(gate), _i(_code(gate) if gate is not None else F32), _i(n), _i(s), _i(w), _stream())
+    return x
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, tok_entry: torch.Tensor, entry_start: torch.Tensor,
+                slots: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = h[t] + (h[t - 1] - h[t]) * mu, where the token before an entry's first comes from state[slot] ([W]
+    float32: zeros at the start of a sequence); state[slot] then takes the entry's last h.  out must not be h."""
+    n, w = h.shape
+    _chk(h, "token_shift.h")
+    _chk(out, "token_shift.out", h.dtype, (n, w))
+    if out.data_ptr() == h.data_ptr():
+        raise KernelError("token_shift: the result needs a buffer of its own")
+    _chk(mu, "token_shift.mu", torch.float32, (w,))
+    _chk(tok_entry, "token_shift.tok_entry", torch.int32, (n,))
+    _chk(entry_start, "token_shift.entry_start", torch.int32)
+    _chk(slots, "token_shift.slots", torch.int32)
+    sp, ss = _state_rows(state, "token_shift", w)
+    _run(load_lib("vt_streams", half=_half(h)), "vt_token_shift", _ptr(h), _i(_code(h)), _ptr(mu), sp, ss, _ptr(tok_entry),
+         _ptr(entry_start), _ptr(slots), _ptr(out), _i(n), _i(w), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+# a feed-forward of many experts (vt_moe.hip)
+def moe_route(x: torch.Tensor, router: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, score: str = "sigmoid",
+              renormalize: bool = False) -> None:
+    """ids[t], weights[t] <- the `top` experts with the largest scores of token t and those scores (the largest
+    first, the lower index among equals); scores are sigmoid or softmax of router x, in float32; renormalize: the
+    chosen scores are divided by their sum.  x [n, W], router [E, W] float32, ids [n, top] int32, weights [n, top]."""
+    n, w = x.shape
+    e = router.shape[0]
+    _chk(x, "moe_route.x")
+    _chk(router, "moe_route.router", torch.float32, (e, w))
+    top = ids.shape[1] if ids.dim() == 2 else 0
+    _chk(ids, "moe_route.ids", torch.int32, (n, top))
+    _chk(weights, "moe_route.weights", torch.float32, (n, top))
+    if score not in ("sigmoid", "softmax") or not 1 <= top <= e:
+        raise KernelError(f"moe_route: score {score!r}, {top} of {e} experts")
+    _run(load_lib("vt_moe", half=_half(x)), "vt_moe_route", _ptr(x), _i(_code(x)), _ptr(router), _ptr(ids), _ptr(weights),
+         _i(n), _i(e), _i(w), _i(top), _i(1 if score == "softmax" else 0), _i(1 if renormalize else 0), _stream())
+
+
+def moe_gate_up(x: torch.Tensor, w_gu: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, act: torch.Tensor,
+                scale_input: bool, alpha: float = 1.0, cubic: float = 0.0) -> torch.Tensor:
+    """act[t * top + k] = f(W_gate,e xe) * (W_up,e xe) for e = ids[t, k], xe = x[t] (times weights[t, k] if
+    scale_input, rounded to x's type), f(g) = g sigmoid(alpha g (1 + cubic g^2)); w_gu [E, 2 F, W] (gate rows, then up
+    rows); act [n * top, F] in x's type.  An expert's matrices are read once per token that chose it."""
+    n, w = x.shape
+    e, two_f, _ = w_gu.shape
+    top = ids.shape[1]
+    _chk(x, "moe_gate_up.x")
+    _chk(w_gu, "moe_gate_up.w_gu", x.dtype, (e, two_f, w))
+    _chk(ids, "moe_gate_up.ids", torch.int32, (n, top))
+    _chk(weights, "moe_gate_up.weights", torch.float32, (n, top))
+    _chk(act, "moe_gate_up.act", x.dtype, (n * top, two_f // 2))
+    _run(load_lib("vt_moe", half=_half(x)), "vt_moe_gate_up", _ptr(x), _i(_code(x)), _ptr(w_gu), _i(_code(w_gu)), _ptr(ids),
+         _ptr(weights), _ptr(act), _i(n), _i(e), _i(w), _i(two_f // 2), _i(top), _i(1 if scale_input else 0), _f(alpha),
+         _f(cubic), _stream())
+    return act
+
+
+def moe_down(act: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, out: torch.Tensor,
+             scale_output: bool) -> torch.Tensor:
+    """out[t] = sum_k (weights[t, k] if scale_output) * W_down,e act[t * top + k], e = ids[t, k], in the order of k;
+    w_down [E, W, F]; out [n, W] float32."""
+    e, w, f = w_down.shape
+    n, top = ids.shape
+    _chk(act, "moe_down.act", None, (n * top, f))
+    _chk(w_down, "moe_down.w_down", act.dtype)
+    _chk(ids, "moe_down.ids", torch.int32)
+    _chk(weights, "moe_down.weights", torch.float32, (n, top))
+    _chk(out, "moe_down.out", torch.float32, (n, w))
+    _run(load_lib("vt_moe", half=_half(act)), "vt_moe_down", _ptr(act), _i(_code(act)), _ptr(w_down), _i(_code(w_down)),
+         _ptr(ids), _ptr(weights), _ptr(out), _i(n), _i(e), _i(w), _i(f), _i(top), _i(1 if scale_output else 0), _stream())
     return out
 
 

@@ -41,13 +41,16 @@ class DecoderModel:
         self.offsets_name: Optional[str] = spec.stream_offsets["name"] if spec.stream_offsets else None
         self.offsets_rows = int(spec.stream_offsets["rows"]) if spec.stream_offsets else 0
         self.offsets: Optional[torch.Tensor] = None
+        # several residual streams: [tokens, streams, width] between the embedding and the final norm
+        self.streams = int(spec.streams)
+        self._stream_ones: Optional[torch.Tensor] = None
 
     def _build_layer(self, ls: LayerSpec, shared: dict):
         rt, width = self.rt, self.spec.hidden_size
         norms = {role: build_part(NORMS, ns, ls.prefix, rt=rt, width=width) for role, ns in ls.norms.items()}
         mixer = build_part(MIXERS, ls.mixer, ls.prefix, rt=rt, width=width, shared=shared)
         ffn = build_part(FEED_FORWARDS, ls.feed_forward, ls.prefix, rt=rt, width=width) if ls.feed_forward is not None else None
-        return BLOCKS.build(ls.block, rt=rt, norms=norms, mixer=mixer, feed_forward=ffn)
+        return build_part(BLOCKS, ls.block, ls.prefix, rt=rt, width=width, norms=norms, mixer=mixer, feed_forward=ffn)
 
     # ------------------------------------------------------------------
     def parts(self) -> List[Part]:
@@ -89,6 +92,9 @@ class DecoderModel:
         """Run the tokens of one step.  caches[i] / states[i] belong to schedule entry i.
         Returns fp32 logits [rows wanted, vocab], or None if no row is wanted."""
         h = self.embedding.forward(ctx.token_ids)
+        if self.streams:
+            # every stream starts as the embedding's output
+            h = ops.streams_fill(h, self.rt.buffer("streams", (h.shape[0], self.streams, h.shape[1]), torch.float32))
         delta = None
         last = len(self.schedule) - 1
         for i, entry in enumerate(self.schedule):
@@ -112,5 +118,11 @@ class DecoderModel:
             return None
         if isinstance(delta, NormedInput):
             delta = None
-        x = self.final_norm.forward(h, delta, rows=ctx.logit_rows)
+        if self.streams:
+            # the streams' sum, for the wanted rows only, inside the final norm's kernel
+            if self._stream_ones is None:
+                self._stream_ones = torch.ones(self.streams, dtype=torch.float32, device=self.rt.device)
+            x = self.final_norm.forward_streams(h, self._stream_ones, rows=ctx.logit_rows)
+        else:
+            x = self.final_norm.forward(h, delta, rows=ctx.logit_rows)
         return self.head.forward(x)

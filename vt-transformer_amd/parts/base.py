@@ -48,7 +48,9 @@ class TensorDecl:
 
     role "matrix": kept in the runtime's dtype (bfloat16, float16 or float32);
     "gain", "bias": small vectors, kept in float32 (exact from bfloat16);
-    "table": integers, kept as int32.  A tensor stored in 32-bit stays so."""
+    "table": integers, kept as int32; "matrix32": a matrix that is kept in float32 whatever the runtime's dtype (a
+    router, whose sums decide which expert a token goes to); "stream_mix": a small square matrix of float32 numbers
+    that lies around the identity.  A tensor stored in 32-bit stays so."""
 
     shape: Tuple[int, ...]
     role: str
@@ -139,7 +141,7 @@ class Runtime:
             if t.dtype in (torch.float32, torch.bfloat16, torch.float16, torch.float64):
                 return t.to(device=self.device, dtype=self.dtype).contiguous()
             raise ValueError(f"matrix of dtype {t.dtype}")
-        if role in ("gain", "bias"):
+        if role in ("gain", "bias", "matrix32", "stream_mix"):
             return t.to(device=self.device, dtype=torch.float32).contiguous()
         if role == "table":
             return t.to(device=self.device, dtype=torch.int32).contiguous()

@@ -17,12 +17,13 @@ part behind the norm then takes as its input.
 """
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import Callable, Dict, Optional, Tuple
 
 import torch
 
-from .base import BLOCKS, NormedInput, Part, Runtime
-from .linear import can_fuse
+from ..kernels import ops
+from .base import BLOCKS, NormedInput, Part, Runtime, StateNeed, TensorDecl
+from .linear import can_fuse, linear
 
 
 @BLOCKS.register("prenorm")
@@ -31,7 +32,7 @@ class PreNormBlock(Part):
     replayable = True
     takes_next_norm = True      # forward(..., next_norm=): the norm that the layer behind this one starts with
 
-    def __init__(self, *, rt: Runtime, norms, mixer, feed_forward):
+    def __init__(self, *, rt: Runtime, norms, mixer, feed_forward, prefix: str = "", width: int = 0):
         self.rt = rt
         self.norm_in = norms["input"]
         self.mixer = mixer
@@ -77,3 +78,127 @@ class PreNormBlock(Part):
             part.forward(x, *args, residual=h)
             return None
         return part.forward(x, *args)
+
+
+@BLOCKS.register("hyper")
+class HyperBlock(Part):
+    """Pre-norm sublayers around S residual streams x_1 .. x_S (float32, [tokens, S, width]) instead of one.  For
+    sublayer q (1: the mixer, 2: the feed-forward) with its learned numbers in_q [S], out_q [S] and mix_q [S, S]:
+
+        u   = sum_s in_q[s] x_s
+        h   = norm_q(u)
+        y   = sublayer(h') * sigmoid(W_rg,q h + b_rg,q)        residual_gate; without it y = sublayer(h')
+        x_t <- sum_s mix_q[s, t] x_s + out_q[t] y              all streams at once from the old ones
+
+    h' is h, or for the mixer with token_shift the blend h + (h_prev - h) * mu with the previous token's h (as it was
+    before blending; zeros in front of a sequence's first token), mu one number per channel.  The previous h of a
+    request's last token is part of its state: the block declares one float32 row per request that holds it in front
+    of whatever the mixer keeps there.  The weighted sum and the norm are one kernel, and so are the gate, the mixing
+    and the addition.  With learned_streams False there is one stream with in = out = mix = 1 and no tensors for
+    them: the plain residual sum.
+    """
+
+    norm_roles = ("input", "post_mixer")
+    replayable = True
+
+    def __init__(self, *, rt: Runtime, norms, mixer, feed_forward, prefix: str = "", width: int = 0, streams: int = 1,
+                 learned_streams: bool = True, token_shift: bool = False, residual_gate: bool = False,
+                 names: Optional[Dict[str, str]] = None):
+        """names: tensor names behind the layer's prefix, with {} standing for the sublayer's number, for in, out, mix
+        (the streams' numbers), gate and gate_bias (the residual gate's matrix and bias), and for shift (mu)."""
+        self.rt, self.width, self.s = rt, int(width), int(streams)
+        if not 1 <= self.s <= ops.STREAMS_MAX:
+            raise ValueError(f"{self.s} residual streams (1 to {ops.STREAMS_MAX})")
+        if not learned_streams and self.s != 1:
+            raise ValueError("streams without learned numbers are one stream")
+        self.learned, self.shift, self.gated = bool(learned_streams), bool(token_shift), bool(residual_gate)
+        self.norm_in = norms["input"]
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norm_post = norms["post_mixer"] if feed_forward is not None else None
+        n = {"in": "hc{}.in", "out": "hc{}.out", "mix": "hc{}.mix", "gate": "rg{}", "gate_bias": "rg{}.b", "shift": "shift"}
+        n.update(names or {})
+        self.names = {k: prefix + v for k, v in n.items()}
+        self.n_sub = 1 if feed_forward is None else 2
+        self.w_in = [None, None]
+        self.w_out = [None, None]
+        self.w_mix = [None, None]
+        self.w_gate, self.p_gate, self.b_gate, self.b_gate_lowp = [None, None], [None, None], [None, None], [None, None]
+        self.mu = None
+        inner = mixer.state_need() if hasattr(mixer, "state_need") else None
+        if inner is not None and (inner.dtype != torch.float32 or len(inner.shape) != 1):
+            raise ValueError("a mixer inside this block keeps its state as one float32 row per request")
+        self.inner_floats = int(inner.shape[0]) if inner is not None else 0
+        self.own_floats = self.width if self.shift else 0
+
+    def parts(self):
+        if self.feed_forward is None:
+            return [self, self.norm_in, self.mixer]
+        return [self, self.norm_in, self.mixer, self.norm_post, self.feed_forward]
+
+    def state_need(self) -> Optional[StateNeed]:
+        """One float32 row per request: the previous token's mixer input (if token_shift), then the mixer's state."""
+        total = self.own_floats + self.inner_floats
+        return StateNeed((total,), torch.float32) if total else None
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        nm, t = self.names, {}
+        for q in range(1, self.n_sub + 1):
+            if self.learned:
+                t[nm["in"].format(q)] = TensorDecl((self.s,), "gain")
+                t[nm["out"].format(q)] = TensorDecl((self.s,), "gain")
+                t[nm["mix"].format(q)] = TensorDecl((self.s, self.s), "stream_mix")
+            if self.gated:
+                t[nm["gate"].format(q)] = TensorDecl((self.width, self.width), "matrix")
+                t[nm["gate_bias"].format(q)] = TensorDecl((self.width,), "bias")
+        if self.shift:
+            t[nm["shift"]] = TensorDecl((self.width,), "bias")
+        return t
+
+    def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
+        nm = self.names
+        for i in range(self.n_sub):
+            q = i + 1
+            if self.learned:
+                self.w_in[i] = rt.place(get(nm["in"].format(q)), "gain")
+                self.w_out[i] = rt.place(get(nm["out"].format(q)), "gain")
+                self.w_mix[i] = rt.place(get(nm["mix"].format(q)), "stream_mix")
+            else:
+                one = torch.ones(1, dtype=torch.float32, device=rt.device)
+                self.w_in[i], self.w_out[i], self.w_mix[i] = one, one, one.view(1, 1)
+            if self.gated:
+                w = rt.place(get(nm["gate"].format(q)), "matrix")
+                self.b_gate[i] = rt.place(get(nm["gate_bias"].format(q)), "bias")
+                self.b_gate_lowp[i] = self.b_gate[i].to(rt.dtype)
+                self.p_gate[i] = rt.pack(w)
+                self.w_gate[i] = rt.row_major(w, self.p_gate[i])
+        if self.shift:
+            self.mu = rt.place(get(nm["shift"]), "bias")
+
+    def _sublayer(self, i: int, part, norm, x, ctx, shift_state, *args):
+        rt = self.rt
+        h = norm.forward_streams(x, self.w_in[i])
+        gate = None
+        if self.gated:
+            gate = linear(rt, h, self.w_gate[i], self.b_gate[i], f"hyper.gate{i}", bias_lowp=self.b_gate_lowp[i],
+                          packed=self.p_gate[i])
+        if shift_state is not None:
+            h = ops.token_shift(h, self.mu, shift_state, ctx.tok_entry, ctx.entry_start, ctx.state_slots,
+                                rt.buffer("hyper.shifted", tuple(h.shape), h.dtype))
+        y = part.forward(h, ctx, *args)
+        ops.streams_write(x, self.w_mix[i], self.w_out[i], y, gate)
+
+    def forward(self, x: torch.Tensor, delta, ctx, cache, state) -> Tuple[torch.Tensor, object]:
+        """x [tokens, S, width] float32, changed in place; nothing is left to be added (`delta` stays None)."""
+        if x.dim() != 3 or x.shape[1] != self.s or delta is not None:
+            raise RuntimeError(f"this block works on {self.s} residual streams [tokens, {self.s}, width]")
+        shift_state = inner_state = None
+        if self.own_floats or self.inner_floats:
+            if state is None or state.dim() != 2 or state.shape[1] != self.own_floats + self.inner_floats:
+                raise RuntimeError("the block was given no state of its shape")
+            shift_state = state[:, :self.own_floats] if self.own_floats else None
+            inner_state = state[:, self.own_floats:] if self.inner_floats else None
+        self._sublayer(0, self.mixer, self.norm_in, x, ctx, shift_state, cache, inner_state)
+        if self.feed_forward is not None:
+            self._sublayer(1, self.feed_forward, self.norm_post, x, ctx, None)
+        return x, None

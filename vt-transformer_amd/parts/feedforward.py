@@ -12,12 +12,15 @@ The gate's form has parameters: with g = gate(x) and u = up(x), both with their
 biases if the model has them,
 
     g <- min(g, limit),  u <- clamp(u, -limit, limit)        (limit 0: no bounds)
-    act = g * sigmoid(alpha * g) * (u + up_shift)
+    act = g * sigmoid(alpha * g * (1 + cubic * g^2)) * (u + up_shift)
 
-alpha 1, no bounds and no shift is SiLU gating, the reference's.
+alpha 1, no bounds, no shift and cubic 0 is SiLU gating, the reference's.  activation "gelu_tanh" is the tanh form of
+GELU, 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))): since (1 + tanh z) / 2 = sigmoid(2 z) it is the same form
+with alpha = 2 sqrt(2 / pi) and cubic = 0.044715.
 """
 from __future__ import annotations
 
+import math
 from typing import Callable, Dict, Optional
 
 import torch
@@ -34,17 +37,23 @@ class GatedMLP(Part):
 
     def __init__(self, *, rt: Runtime, width: int, prefix: str, intermediate_size: int, activation: str = "silu",
                  names: Optional[Dict[str, str]] = None, weight_suffix: str = ".weight",
-                 bias_suffix: Optional[str] = None, act_alpha: float = 1.0, act_limit: float = 0.0, up_shift: float = 0.0):
+                 bias_suffix: Optional[str] = None, act_alpha: float = 1.0, act_limit: float = 0.0, up_shift: float = 0.0,
+                 act_cubic: float = 0.0):
         """names: the three matrices' names behind the prefix; weight_suffix: what follows a matrix's name in its
         tensor's name ("" where the tensor is called as the matrix); bias_suffix: likewise for the three biases
-        (None: the projections have none); act_alpha, act_limit, up_shift: the gate's form (module docstring)."""
-        if activation != "silu":
-            raise ValueError(f"activation '{activation}' is not supported (only 'silu', whose form act_alpha, act_limit "
-                             f"and up_shift change)")
+        (None: the projections have none); activation: "silu" or "gelu_tanh"; act_alpha, act_limit, up_shift, act_cubic:
+        the gate's form (module docstring; "gelu_tanh" sets alpha and cubic itself)."""
+        if activation == "gelu_tanh":
+            if act_alpha != 1.0 or act_cubic != 0.0:
+                raise ValueError("activation 'gelu_tanh' fixes act_alpha and act_cubic")
+            act_alpha, act_cubic = 2.0 * math.sqrt(2.0 / math.pi), 0.044715
+        elif activation != "silu":
+            raise ValueError(f"activation '{activation}' is not supported ('silu', whose form act_alpha, act_limit, "
+                             f"up_shift and act_cubic change, and 'gelu_tanh' are)")
         if not act_alpha > 0 or act_limit < 0:
             raise ValueError("act_alpha must be positive and act_limit not negative (0: no bounds)")
-        self.alpha, self.limit, self.shift = float(act_alpha), float(act_limit), float(up_shift)
-        self.plain_silu = self.alpha == 1.0 and self.limit == 0.0 and self.shift == 0.0
+        self.alpha, self.limit, self.shift, self.cubic = float(act_alpha), float(act_limit), float(up_shift), float(act_cubic)
+        self.plain_silu = self.alpha == 1.0 and self.limit == 0.0 and self.shift == 0.0 and self.cubic == 0.0
         self.bias_suffix = bias_suffix
         self.b_gu = self.b_gu_lowp = self.b_down = self.b_down_lowp = None
         self.rt = rt
@@ -105,15 +114,15 @@ class GatedMLP(Part):
                     x, normed = x.materialize(), False
             if normed and x.prepared:
                 ops.gated_linear_bf16_form(x.xn, self.p_gu, self.b_gu, act, self.alpha, self.limit, self.shift,
-                                           norm_eps=x.eps, ssq_in=x.ssq)
+                                           norm_eps=x.eps, ssq_in=x.ssq, cubic=self.cubic)
             elif normed:
                 ops.gated_linear_bf16_form(x.h, self.p_gu, self.b_gu, act, self.alpha, self.limit, self.shift,
-                                           norm_gain=x.gain, norm_eps=x.eps)
+                                           norm_gain=x.gain, norm_eps=x.eps, cubic=self.cubic)
             else:
-                ops.gated_linear_bf16_form(x, self.p_gu, self.b_gu, act, self.alpha, self.limit, self.shift)
+                ops.gated_linear_bf16_form(x, self.p_gu, self.b_gu, act, self.alpha, self.limit, self.shift, cubic=self.cubic)
         else:
             gu = linear(rt, x, self.w_gu, self.b_gu, "mlp.gu", bias_lowp=self.b_gu_lowp)
-            ops.gated_act(gu, act, self.alpha, self.limit, self.shift)
+            ops.gated_act(gu, act, self.alpha, self.limit, self.shift, self.cubic)
         return linear(rt, act, self.w_down, self.b_down, "mlp.down", bias_lowp=self.b_down_lowp, packed=self.p_down,
                       residual=residual, hand_on=hand_on)
 

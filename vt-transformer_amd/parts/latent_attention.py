@@ -6,7 +6,8 @@ Per token, from the mixer's input x:
     q_h = [qn_h (plain_dim) | qr_h (rot_dim)]       = rows of W_q x, head by head
     [c_raw (rank) | kr (rot_dim)]                   = W_dkv x
     c  = c_raw / rms(c_raw) * w_norm                 (eps inside the root)
-    qr_h, kr rotated by position (the leading rot.dim elements, half-split pairs); kr is shared by all heads
+    qr_h, kr rotated by position (the leading rot.dim elements; element i with i + rot.dim/2, or with rot_pairs =
+    "neighbours" element 2i with 2i + 1); kr is shared by all heads
     k_h = [W_uk,h c | kr],  v_h = W_uv,h c
     score_h(i, j) = scale * q_h(i) . k_h(j),  j seen from i  <=>  0 <= i - j < window (window 0: every j <= i)
     p = softmax over the seen keys, with exp(sink_h) added to the denominator if the mixer has sinks
@@ -40,13 +41,19 @@ class LatentAttention(Part):
     def __init__(self, *, rt: Runtime, width: int, prefix: str, num_heads: int, plain_dim: int, rot_dim: int,
                  value_dim: int, rank: int, norm_eps: float, position: Optional[PartSpec] = None,
                  scale: Optional[float] = None, window: int = 0, sink: bool = False, out_gate: bool = False,
-                 shared: Optional[dict] = None, names: Optional[Dict[str, str]] = None):
+                 shared: Optional[dict] = None, names: Optional[Dict[str, str]] = None, rot_pairs: str = "halves"):
         """plain_dim / rot_dim: a query head's unrotated and rotated elements; value_dim: a head's values; rank: the
         low-rank vector's size; norm_eps: eps of its RMS norm; position: a rotary encoding of at most rot_dim
         elements (None: nothing is rotated); window: 0 or how many positions back a token sees, itself included;
         sink: a learned number per head in the softmax's denominator; out_gate: the heads' outputs times
         sigmoid(W_g x), element by element; names: tensor names behind the prefix for q, dkv, dkv_norm, uk, uv, o,
-        g, sink."""
+        g, sink; rot_pairs: which elements of the rotated part turn together, "halves" (i with i + dims/2) or
+        "neighbours" (2i with 2i + 1).  A score is a sum over the elements of q and k alike, so neighbours are
+        served by the same kernels: the rows of W_q and W_dkv that make the rotated parts are put into the
+        half-split order once, when they are loaded (pair i's two elements to places i and i + dims/2)."""
+        if rot_pairs not in ("halves", "neighbours"):
+            raise ValueError(f"rot_pairs '{rot_pairs}' is not known ('halves' and 'neighbours' are)")
+        self.rot_pairs = rot_pairs
         self.rt, self.width = rt, int(width)
         self.nh, self.dn, self.dr = int(num_heads), int(plain_dim), int(rot_dim)
         self.dv, self.rank = int(value_dim), int(rank)
@@ -120,6 +127,15 @@ class LatentAttention(Part):
     def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
         nm = self.names
         mats = [rt.place(get(nm[k]), "matrix") for k in (("q", "dkv", "g") if self.out_gate else ("q", "dkv"))]
+        dims = int(getattr(self.position, "dim", 0))
+        if self.rot_pairs == "neighbours" and dims:
+            # rows of the rotated parts: pair i's elements from places 2i and 2i + 1 to places i and i + dims/2
+            order = torch.cat([torch.arange(0, dims, 2), torch.arange(1, dims, 2), torch.arange(dims, self.dr)]).to(mats[0].device)
+            per_head = self.dn + self.dr
+            q_rows = torch.cat([torch.cat([torch.arange(self.dn, device=order.device), self.dn + order]) + h * per_head
+                                for h in range(self.nh)])
+            mats[0] = mats[0].index_select(0, q_rows)
+            mats[1] = mats[1].index_select(0, torch.cat([torch.arange(self.rank, device=order.device), self.rank + order]))
         self.w_in = torch.cat(mats, dim=0).contiguous()
         self.w_o = rt.place(get(nm["o"]), "matrix")
         # W_uk is only ever used transposed (queries go through it, not the cache): kept as [H][rank][plain_dim], so

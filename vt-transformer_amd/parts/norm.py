@@ -23,19 +23,32 @@ class RMSNorm(Part):
     # the way (NormedInput); any norm of that form may say so
     rms_fusable = True
 
-    def __init__(self, *, rt: Runtime, width: int, prefix: str, eps: float, name: str = "weight", scratch: str = "norm"):
+    def __init__(self, *, rt: Runtime, width: int, prefix: str, eps: float, name: str = "weight", scratch: str = "norm",
+                 unit_offset: bool = False):
+        """unit_offset: the tensor holds w = gain - 1 (the one is added once, in float32, when it is loaded)."""
         self.rt = rt
         self.width = int(width)
         self.eps = float(eps)
         self.name = prefix + name
         self.scratch = scratch
+        self.unit_offset = bool(unit_offset)
         self.gain: Optional[torch.Tensor] = None
 
     def tensors(self) -> Dict[str, TensorDecl]:
-        return {self.name: TensorDecl((self.width,), "gain")}
+        # (a gain less one is drawn like a bias where a model gets random weights)
+        return {self.name: TensorDecl((self.width,), "bias" if self.unit_offset else "gain")}
 
     def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
         self.gain = rt.place(get(self.name), "gain")
+        if self.unit_offset:
+            self.gain = (self.gain + 1.0).contiguous()
+
+    def forward_streams(self, x: torch.Tensor, w_in: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The norm of a weighted sum of several residual streams: x [N, S, H] float32, w_in [S] float32 -> normed
+        [N or R, H] in the runtime's dtype (one kernel: the sum is never written)."""
+        n = rows.numel() if rows is not None else x.shape[0]
+        out = self.rt.buffer(self.scratch + (".rows" if rows is not None else ""), (n, self.width), self.rt.dtype)
+        return ops.streams_read(x, w_in, self.gain, out, self.eps, rows=rows)
 
     def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor] = None,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:

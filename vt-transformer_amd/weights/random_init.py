@@ -76,12 +76,17 @@ def random_tensor(name: str, decl: TensorDecl, seed: int, device: torch.device, 
     if torch.device(device).type == "cuda":
         from ..kernels import ops
         out = torch.empty(decl.shape, dtype=dtype, device=device)
-        return ops.random_normal(out, key, normal_scale(STD), mean)
-    out = torch.empty(n, dtype=dtype)
-    for first in range(0, n, _HOST_PIECE):
-        m = min(_HOST_PIECE, n - first)
-        out[first:first + m] = torch.from_numpy(counter_normal(key, first, m, STD, mean)).to(dtype)
-    return out.reshape(decl.shape)
+        out = ops.random_normal(out, key, normal_scale(STD), mean)
+    else:
+        out = torch.empty(n, dtype=dtype)
+        for first in range(0, n, _HOST_PIECE):
+            m = min(_HOST_PIECE, n - first)
+            out[first:first + m] = torch.from_numpy(counter_normal(key, first, m, STD, mean)).to(dtype)
+        out = out.reshape(decl.shape)
+    if decl.role == "stream_mix":
+        # a small square matrix around the identity (the deviates, rounded as every other tensor, plus the ones)
+        out = (out.to(torch.float32) + torch.eye(decl.shape[0], dtype=torch.float32, device=out.device)).to(dtype)
+    return out
 
 
 def random_tensors(expected: Dict[str, TensorDecl], seed: int, device: torch.device,
