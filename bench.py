@@ -211,6 +211,29 @@ def gabelorn_pair_configs(key: str, window: int):
     return gab, qwen
 
 
+def kigalix_pair_configs(key: str, streams: int):
+    """(Kigalix config.json, Gabelorn config.json) of equal sizes.  Kigalix: general-delta, latent-attention and gated
+    latent-attention layers in turn over `streams` residual streams; a dense feed-forward and a mixture of eight
+    experts (two per token, a quarter of the dense size each) take turns behind them.  Its latent layers keep
+    Gabelorn's 192 + 64 numbers per token and see every key; the delta layers have heads of 64.  Gabelorn: the
+    pair of `gabelorn_pair_configs` with a window that no prompt of the run reaches."""
+    width, layers, heads, kv, d, ff, vocab = PAIR_SIZES[key]
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2}}
+    lat = {"heads": heads, "dim": d, "rot_dim": 64, "vdim": d, "kv_rank": 192, "scale": (d + 64) ** -0.5}
+    mixers = [
+        ("general_delta", {"heads": width // 64, "dim": 64, "decay_rank": 64}),
+        ("latent_attention", dict(lat, rot={"dims": 64, "base": 1e6})),
+        ("latent_attention_2", dict(lat, rot={"dims": 64, "base": 1e6, "scaling": {"factor": 8.0, "original": 4096,
+                                                                                   "fast": 32.0, "slow": 1.0}})),
+    ]
+    kig = {"architecture": "Kigalix", "vocab": vocab, "width": width, "streams": streams, "norm": {"eps": 1e-6},
+           "layers": [{"type": mixers[i % 3][0], "mixer": mixers[i % 3][1], "mlp": dense if i % 2 == 0 else moe}
+                      for i in range(layers)], "max_positions": 32768}
+    gab, _ = gabelorn_pair_configs(key, 32768)
+    return kig, gab
+
+
 class PairBench(Bench):
     """Bench's measurements on an engine built from any config.json."""
 
@@ -233,8 +256,10 @@ class PairBench(Bench):
 
 
 def design_pairs(args, design: str) -> int:
-    """Prefill and decode of a second design (lisunex or gabelorn) beside Qwen2 at equal sizes; one JSON line."""
+    """Prefill and decode of a second design (lisunex or gabelorn beside Qwen2, kigalix beside Gabelorn) at equal
+    sizes; one JSON line."""
     title = design.capitalize()
+    beside = "gabelorn" if design == "kigalix" else "qwen2"
     keys = [k.strip() for k in getattr(args, design).split(",") if k.strip()]
     for k in keys:
         if k not in PAIR_SIZES:
@@ -243,33 +268,41 @@ def design_pairs(args, design: str) -> int:
     T, batch, prompt_len = args.prefill_tokens, args.batch, args.prompt_len or 1024
     per_req = -(-(prompt_len + args.steps + args.warmup + 32) // 16) * 16
     pool = max(batch * per_req, T + 64)
-    span = args.lisunex_chunk if design == "lisunex" else args.gabelorn_window
+    span = {"lisunex": args.lisunex_chunk, "gabelorn": args.gabelorn_window, "kigalix": args.kigalix_streams}[design]
+    make = {"lisunex": pair_configs, "gabelorn": gabelorn_pair_configs, "kigalix": kigalix_pair_configs}[design]
+    only = getattr(args, "only", "")
     out = {}
     for k in keys:
-        other, qwen = pair_configs(k, span) if design == "lisunex" else gabelorn_pair_configs(k, span)
+        other, qwen = make(k, span)
         row = {}
-        for name, cfg_d in ((design, other), ("qwen2", qwen)):
+        for name, cfg_d in ((design, other), (beside, qwen)):
+            if only and name != only:
+                continue
             b = PairBench(f"{name} {k}", cfg_d, args.dtype, batch, pool, max(pool // batch, T + 64) + 64, graphs=not args.no_graphs)
             p_dt = b.prefill_run(T)
             tps, ms, _ = b.decode_run(batch, args.steps, args.warmup, prompt_len)
             row[name] = {"prefill_tok_s": round(T / p_dt, 1), "prefill_ms": round(p_dt * 1e3, 3),
                          "decode_tok_s": round(tps, 1), "decode_ms_per_step": round(ms, 4)}
             b.close()
-        row[f"{design}_over_qwen2"] = {"prefill": round(row[design]["prefill_tok_s"] / row["qwen2"]["prefill_tok_s"], 3),
-                                       "decode": round(row[design]["decode_tok_s"] / row["qwen2"]["decode_tok_s"], 3)}
+        if design in row and beside in row:
+            row[f"{design}_over_{beside}"] = {"prefill": round(row[design]["prefill_tok_s"] / row[beside]["prefill_tok_s"], 3),
+                                              "decode": round(row[design]["decode_tok_s"] / row[beside]["decode_tok_s"], 3)}
         width, layers, heads, kv, d, ff, vocab = PAIR_SIZES[k]
         row["sizes"] = f"L{layers} H{width} NH{heads} KVH{kv} D{d} I{ff} V{vocab}"
         out[k] = row
     first = out[keys[0]]
+    if design not in first:
+        first = dict(first, **{design: first[beside]})
     print(json.dumps({
         "metric": f"{title} decode tok/s at batch {batch} after {prompt_len:,}-token prompts, sizes {keys[0]} "
-                  f"(beside Qwen2 at equal sizes; prefill of {T:,} tokens under `pairs`)",
+                  f"(beside {beside.capitalize()} at equal sizes; prefill of {T:,} tokens under `pairs`)",
         "value": first[design]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": first[design]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": {"bfloat16": "bf16", "float16": "fp16"}[args.dtype],
         "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
-        "config": {"model": f"{title} and Qwen2 at equal sizes", "global_batch": batch, "seq_len": prompt_len,
-                   "prefill_tokens": T, "chunk" if design == "lisunex" else "window": span, "parallelism": "1 GPU"},
+        "config": {"model": f"{title} and {beside.capitalize()} at equal sizes", "global_batch": batch, "seq_len": prompt_len,
+                   "prefill_tokens": T, {"lisunex": "chunk", "gabelorn": "window", "kigalix": "streams"}[design]: span,
+                   "parallelism": "1 GPU"},
         "pairs": out}), flush=True)
     return 0
 
@@ -322,15 +355,23 @@ def main() -> int:
                          "turn) beside Qwen2 at equal sizes, prefill of --prefill-tokens and decode at --batch; sizes by "
                          "name, with commas: " + ", ".join(PAIR_SIZES))
     ap.add_argument("--gabelorn-window", type=int, default=1024, help="positions that a latent-attention layer sees")
+    ap.add_argument("--kigalix", default="", metavar="SIZES",
+                    help="another workload instead: the Kigalix design (general-delta and latent-attention layers over "
+                         "several residual streams, dense and expert feed-forwards in turn) beside Gabelorn at equal "
+                         "sizes, prefill of --prefill-tokens and decode at --batch; sizes by name, with commas: "
+                         + ", ".join(PAIR_SIZES))
+    ap.add_argument("--kigalix-streams", type=int, default=4, help="residual streams of the Kigalix model")
+    ap.add_argument("--only", default="", metavar="MODEL",
+                    help="with --lisunex, --gabelorn or --kigalix: measure one model of the pair alone (profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; N > 1 is not measured")
         return 2
 
-    if args.lisunex or args.gabelorn:
+    if args.lisunex or args.gabelorn or args.kigalix:
         if args.dtype == "float16":
             args.dtype = "bfloat16"         # the serving dtype of these designs
-        return design_pairs(args, "lisunex" if args.lisunex else "gabelorn")
+        return design_pairs(args, "lisunex" if args.lisunex else "gabelorn" if args.gabelorn else "kigalix")
 
     import torch
 

@@ -68,13 +68,82 @@ __global__ __launch_bounds__(256) void streams_read_kernel(const float* __restri
     }
 }
 
+// The same for widths that are multiples of 4 up to 1024 NV: a thread keeps its NV pieces of four sums in registers
+// between the two passes, so the streams are read once, 16 bytes at a time, with all of a thread's loads in flight
+// together.  The weighted sums are those of the kernel above; the sum of squares takes its terms in this layout's order
+// (which of the two kernels runs depends on the width alone).
+template <typename TO, int NV>
+__global__ __launch_bounds__(256) void streams_read_vec_kernel(const float* __restrict__ x, const float* __restrict__ w_in,
+                                                               const float* __restrict__ gain, const int* __restrict__ rows,
+                                                               TO* __restrict__ out, int S, int W, float eps) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const int t = rows ? rows[r] : r;
+    const int W4 = W >> 2;
+    const float4* xt = (const float4*)(x + (size_t)t * S * W);
+    float4 u[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) u[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s = 0; s < S; ++s) {
+        const float wi = w_in[s];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int j = threadIdx.x + 256 * i;
+            if (j < W4) {
+                const float4 v = xt[(size_t)s * W4 + j];
+                u[i].x = fmaf(wi, v.x, u[i].x);
+                u[i].y = fmaf(wi, v.y, u[i].y);
+                u[i].z = fmaf(wi, v.z, u[i].z);
+                u[i].w = fmaf(wi, v.w, u[i].w);
+            }
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        ss = fmaf(u[i].x, u[i].x, ss);
+        ss = fmaf(u[i].y, u[i].y, ss);
+        ss = fmaf(u[i].z, u[i].z, ss);
+        ss = fmaf(u[i].w, u[i].w, ss);
+    }
+    ss = block_sum(ss, red);
+    const float rinv = 1.0f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int j = threadIdx.x + 256 * i;
+        if (j < W4) {
+            const float4 gn = ((const float4*)gain)[j];
+            const float a = (gn.x * u[i].x) * rinv, b = (gn.y * u[i].y) * rinv, c = (gn.z * u[i].z) * rinv, d = (gn.w * u[i].w) * rinv;
+            if constexpr (sizeof(TO) == 4) {
+                ((float4*)out)[(size_t)r * W4 + j] = make_float4(a, b, c, d);
+            } else {
+                uint2 o;
+                o.x = vt_pack2(a, b);
+                o.y = vt_pack2(c, d);
+                ((uint2*)out)[(size_t)r * W4 + j] = o;
+            }
+        }
+    }
+}
+
+template <typename TO>
+static void streams_read_launch(const float* x, const float* w_in, const float* gain, const int* rows, TO* out, int n_out, int S,
+                                int W, float eps, hipStream_t stream) {
+    const bool vec = W % 4 == 0 && W <= 8192 && !(((uintptr_t)x | (uintptr_t)gain | (uintptr_t)out) & 15);
+    if (vec && W <= 1024) streams_read_vec_kernel<TO, 1><<<n_out, 256, 0, stream>>>(x, w_in, gain, rows, out, S, W, eps);
+    else if (vec && W <= 2048) streams_read_vec_kernel<TO, 2><<<n_out, 256, 0, stream>>>(x, w_in, gain, rows, out, S, W, eps);
+    else if (vec && W <= 4096) streams_read_vec_kernel<TO, 4><<<n_out, 256, 0, stream>>>(x, w_in, gain, rows, out, S, W, eps);
+    else if (vec) streams_read_vec_kernel<TO, 8><<<n_out, 256, 0, stream>>>(x, w_in, gain, rows, out, S, W, eps);
+    else streams_read_kernel<TO><<<n_out, 256, 0, stream>>>(x, w_in, gain, rows, out, S, W, eps);
+}
+
 extern "C" int vt_streams_read(const float* x, const float* w_in, const float* gain, const int* rows, void* out,
                                int out_dtype, int n_out, int S, int W, float eps, hipStream_t stream) {
     VT_REQUIRE(n_out >= 0 && W > 0, "vt_streams_read: bad sizes n=%d W=%d", n_out, W);
     VT_REQUIRE(S >= 1 && S <= STREAMS_MAX, "vt_streams_read: %d streams (1 to %d)", S, STREAMS_MAX);
     if (n_out == 0) return 0;
-    if (out_dtype == VT_F32) streams_read_kernel<float><<<n_out, 256, 0, stream>>>(x, w_in, gain, rows, (float*)out, S, W, eps);
-    else if (out_dtype == VT_BF16) streams_read_kernel<bf16_t><<<n_out, 256, 0, stream>>>(x, w_in, gain, rows, (bf16_t*)out, S, W, eps);
+    if (out_dtype == VT_F32) streams_read_launch<float>(x, w_in, gain, rows, (float*)out, n_out, S, W, eps, stream);
+    else if (out_dtype == VT_BF16) streams_read_launch<bf16_t>(x, w_in, gain, rows, (bf16_t*)out, n_out, S, W, eps, stream);
     else return vt_fail("vt_streams_read: unknown out dtype %d", out_dtype);
     VT_CHECK_LAUNCH("vt_streams_read");
     return 0;

@@ -1302,6 +1302,71 @@ def moe_down(act: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, weights
     return out
 
 
+MOE_GROUPED_MAX_EXPERTS = 1024
+MOE_TILE_PAIRS = 128        # pairs of one expert that a block of the grouped products takes
+
+
+def moe_plan_size(pairs: int, experts: int) -> int:
+    """int32 elements of the plan that moe_sort writes for `pairs` (token, choice) pairs."""
+    tiles = -(-int(pairs) // MOE_TILE_PAIRS) + int(experts)         # what vt_moe_plan_tiles says
+    return 1 + int(pairs) + 3 * tiles
+
+
+def moe_grouped_ok(x: torch.Tensor, experts: int, width: int, inter: int) -> bool:
+    """Whether the grouped products take this feed-forward: a 16-bit type, sizes that are multiples of 8."""
+    return x.dtype in LOWP and width % 8 == 0 and inter % 8 == 0 and experts <= MOE_GROUPED_MAX_EXPERTS
+
+
+def moe_sort(ids: torch.Tensor, plan: torch.Tensor, experts: int) -> torch.Tensor:
+    """plan <- the pairs in the order of their experts, cut into tiles of pairs of one expert (what the grouped
+    products read).  ids [n, top] int32 with values below `experts`; plan: moe_plan_size(n * top, experts) int32."""
+    _chk(ids, "moe_sort.ids", torch.int32)
+    pairs = ids.numel()
+    _chk(plan, "moe_sort.plan", torch.int32, (moe_plan_size(pairs, experts),))
+    _run(load_lib("vt_moe"), "vt_moe_sort", _ptr(ids), _ptr(plan), _i(pairs), _i(experts), _stream())
+    return plan
+
+
+def moe_gate_up_grouped(x: torch.Tensor, w_gu: torch.Tensor, plan: torch.Tensor, weights: torch.Tensor, act: torch.Tensor,
+                        top: int, scale_input: bool, alpha: float = 1.0, cubic: float = 0.0) -> torch.Tensor:
+    """moe_gate_up on the matrix cores for many tokens: act [n * top, F] in the plan's order (pairs sorted by expert),
+    an expert's matrices read once per tile of pairs.  x [n, W] and w_gu [E, 2 F, W] of one 16-bit type."""
+    n, w = x.shape
+    e, two_f, _ = w_gu.shape
+    _chk(x, "moe_gate_up_grouped.x")
+    if x.dtype not in LOWP:
+        raise KernelError("moe_gate_up_grouped: a 16-bit type is needed")
+    _chk(w_gu, "moe_gate_up_grouped.w_gu", x.dtype, (e, two_f, w))
+    _chk(plan, "moe_gate_up_grouped.plan", torch.int32, (moe_plan_size(n * top, e),))
+    _chk(weights, "moe_gate_up_grouped.weights", torch.float32, (n, top))
+    _chk(act, "moe_gate_up_grouped.act", x.dtype, (n * top, two_f // 2))
+    _run(load_lib("vt_moe", half=_half(x)), "vt_moe_gate_up_grouped", _ptr(x), _ptr(w_gu), _ptr(plan), _ptr(weights), _ptr(act),
+         _i(n), _i(e), _i(w), _i(two_f // 2), _i(top), _i(1 if scale_input else 0), _f(alpha), _f(cubic), _stream())
+    return act
+
+
+def moe_down_grouped(act: torch.Tensor, w_down: torch.Tensor, plan: torch.Tensor, weights: torch.Tensor, out: torch.Tensor,
+                     scratch: Optional[torch.Tensor], scale_output: bool) -> torch.Tensor:
+    """moe_down on the matrix cores from activations in the plan's order; scratch [n * top, W] float32 where a token
+    has more than one choice (the choices' results, added in their order afterwards)."""
+    e, w, f = w_down.shape
+    n, top = weights.shape
+    _chk(act, "moe_down_grouped.act", None, (n * top, f))
+    if act.dtype not in LOWP:
+        raise KernelError("moe_down_grouped: a 16-bit type is needed")
+    _chk(w_down, "moe_down_grouped.w_down", act.dtype)
+    _chk(plan, "moe_down_grouped.plan", torch.int32, (moe_plan_size(n * top, e),))
+    _chk(weights, "moe_down_grouped.weights", torch.float32)
+    _chk(out, "moe_down_grouped.out", torch.float32, (n, w))
+    if top > 1:
+        if scratch is None:
+            raise KernelError("moe_down_grouped: several choices per token need scratch")
+        _chk(scratch, "moe_down_grouped.scratch", torch.float32, (n * top, w))
+    _run(load_lib("vt_moe", half=_half(act)), "vt_moe_down_grouped", _ptr(act), _ptr(w_down), _ptr(plan), _ptr(weights), _ptr(out),
+         _ptr(scratch if top > 1 else None), _i(n), _i(e), _i(w), _i(f), _i(top), _i(1 if scale_output else 0), _stream())
+    return out
+
+
 # ---------------------------------------------------------------------------
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
            uniform: torch.Tensor, work: torch.Tensor, out: torch.Tensor,

@@ -53,6 +53,8 @@ class ExpertMixture(Part):
         n.update(names or {})
         self.names = {k: prefix + v for k, v in n.items()}
         self.router = self.w_gu = self.w_down = None
+        # pairs (token, choice) from which the experts' products run grouped on the matrix cores
+        self.grouped_from = 16
 
     def tensors(self) -> Dict[str, TensorDecl]:
         nm = self.names
@@ -82,6 +84,12 @@ class ExpertMixture(Part):
         wts = rt.buffer("moe.weights", (n, self.top), torch.float32)
         ops.moe_route(x, self.router, ids, wts, self.score, self.renormalize)
         act = rt.buffer("moe.act", (n * self.top, self.inter), rt.dtype)
-        ops.moe_gate_up(x, self.w_gu, ids, wts, act, self.weight_on == "input", self.alpha, self.cubic)
         out = rt.buffer("moe.out", (n, self.width), torch.float32)
+        if n * self.top >= self.grouped_from and ops.moe_grouped_ok(x, self.ne, self.width, self.inter):
+            plan = rt.buffer("moe.plan", (ops.moe_plan_size(n * self.top, self.ne),), torch.int32)
+            ops.moe_sort(ids, plan, self.ne)
+            ops.moe_gate_up_grouped(x, self.w_gu, plan, wts, act, self.top, self.weight_on == "input", self.alpha, self.cubic)
+            scratch = rt.buffer("moe.choices", (n * self.top, self.width), torch.float32) if self.top > 1 else None
+            return ops.moe_down_grouped(act, self.w_down, plan, wts, out, scratch, self.weight_on == "output")
+        ops.moe_gate_up(x, self.w_gu, ids, wts, act, self.weight_on == "input", self.alpha, self.cubic)
         return ops.moe_down(act, self.w_down, ids, wts, out, self.weight_on == "output")
