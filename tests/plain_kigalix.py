@@ -134,10 +134,17 @@ def dense_mlp(x: torch.Tensor, w: Dict[str, torch.Tensor], p: str) -> torch.Tens
     return (gelu_tanh(x @ w[p + "gate"].T) * (x @ w[p + "up"].T)) @ w[p + "down"].T
 
 
-def expert_mixture(x: torch.Tensor, w: Dict[str, torch.Tensor], p: str, experts: int, top: int) -> torch.Tensor:
+def expert_mixture(x: torch.Tensor, w: Dict[str, torch.Tensor], p: str, experts: int, top: int,
+                   margins: Optional[list] = None) -> torch.Tensor:
     """Every token goes to the `top` experts with the largest sigmoid scores; a chosen expert's score multiplies its
-    input, and the experts' outputs are added."""
-    scores = torch.sigmoid(x @ w[p + "router"].T)
+    input, and the experts' outputs are added.  margins: a list that receives, per token, how far the last chosen
+    expert's logit lies above the first one left out, in units of the logits' spread (a choice that rounding may turn
+    has a small one)."""
+    logits = x @ w[p + "router"].T
+    scores = torch.sigmoid(logits)
+    if margins is not None and top < experts:
+        ranked = torch.sort(logits, dim=-1, descending=True).values
+        margins.append((ranked[:, top - 1] - ranked[:, top]) / logits.std(dim=-1).clamp_min(1e-30))
     out = torch.zeros_like(x)
     chosen = torch.topk(scores, top, dim=-1).indices
     for t in range(x.shape[0]):
@@ -148,9 +155,10 @@ def expert_mixture(x: torch.Tensor, w: Dict[str, torch.Tensor], p: str, experts:
     return out
 
 
-def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], streams: Optional[list] = None) -> torch.Tensor:
+def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], streams: Optional[list] = None,
+            margins: Optional[list] = None) -> torch.Tensor:
     """Logits [T, vocab] of one sequence from position 0.  streams: a list that receives the sum of the residual
-    streams after every layer."""
+    streams after every layer; margins: a list that receives every expert layer's margins (expert_mixture)."""
     w = {k: v.to(DT) for k, v in w.items()}
     eps = float(cfg["norm"]["eps"])
     n_streams = int(cfg.get("streams", 1))
@@ -161,10 +169,14 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], streams: Opti
     def sublayer(q: int, p: str, fn):
         nonlocal xs
         hc = f"{p}hc{q}."
-        read = sum(w[hc + "in"][s] * xs[s] for s in range(n_streams))
+        if "streams" in cfg:
+            w_in, w_out, w_mix = w[hc + "in"], w[hc + "out"], w[hc + "mix"]
+        else:                                   # one stream and no numbers for it: x <- x + y
+            w_in, w_out, w_mix = torch.ones(1, dtype=DT), torch.ones(1, dtype=DT), torch.ones(1, 1, dtype=DT)
+        read = sum(w_in[s] * xs[s] for s in range(n_streams))
         h = offset_rmsnorm(read, w[f"{p}norm{q}"], eps)
         y = fn(h) * torch.sigmoid(h @ w[f"{p}rg{q}"].T + w[f"{p}rg{q}.b"])
-        xs = [sum(w[hc + "mix"][s, t] * xs[s] for s in range(n_streams)) + w[hc + "out"][t] * y for t in range(n_streams)]
+        xs = [sum(w_mix[s, t] * xs[s] for s in range(n_streams)) + w_out[t] * y for t in range(n_streams)]
 
     for i, layer in enumerate(cfg["layers"]):
         p = f"l{i}."
@@ -181,7 +193,8 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], streams: Opti
             if mlp["kind"] == "dense":
                 sublayer(2, p, lambda h: dense_mlp(h, w, p + "mlp."))
             elif mlp["kind"] == "moe":
-                sublayer(2, p, lambda h: expert_mixture(h, w, p + "mlp.", int(mlp["router"]["experts"]), int(mlp["router"]["top"])))
+                sublayer(2, p, lambda h: expert_mixture(h, w, p + "mlp.", int(mlp["router"]["experts"]), int(mlp["router"]["top"]),
+                                                     margins))
             else:
                 raise ValueError(f"feed-forward kind {mlp['kind']!r}")
         if streams is not None:

@@ -61,7 +61,14 @@ def test_declared_tensors():
     assert t["l0.mlp.e4.gate"].shape == (40, 96) and t["l0.mlp.e0.down"].shape == (96, 40) and "l0.mlp.e5.up" not in t
     assert t["l1.mix.q"].shape == (4 * 32, 96) and t["l1.mix.dkv"].shape == (48, 96) and t["l1.mix.dkv.norm"].shape == (32,)
     assert t["l1.mix.uk"].shape == (64, 32) and t["l1.mix.uv"].shape == (96, 32) and "l1.mix.g" not in t
-    assert t["l2.mix.g"].shape == (30, 96) and "l2.norm2" not in t and "l2.hc2.in" not in t and "l2.rg2" not in t
+    # a layer without a feed-forward: the second sublayer's tensors are tolerated in a checkpoint, never required
+    assert t["l2.mix.g"].shape == (30, 96) and all(t[n].optional for n in ("l2.norm2", "l2.hc2.in", "l2.hc2.mix", "l2.rg2", "l2.rg2.b"))
+    assert not t["l2.hc1.in"].optional and not t["l1.hc2.in"].optional and not t["l1.norm2"].optional
+    from vt_transformer_amd.weights.loader import check_tensors
+    for idle in (False, True):
+        held = {n: (w.dtype, tuple(w.shape)) for n, w in make_weights(CFG_A, 1, idle=idle).items()}
+        assert ("l2.norm2" in held) == idle
+        check_tensors(t, held, "here")
     assert t["l1.hc1.in"].shape == (3,) and t["l1.hc2.out"].shape == (3,) and t["l1.hc1.mix"].shape == (3, 3)
     assert t["l1.shift"].shape == (96,) and t["l1.rg1"].shape == (96, 96) and t["l1.rg2.b"].shape == (96,)
     c = declared_tensors(config_from_dict(copy.deepcopy(CFG_C)))

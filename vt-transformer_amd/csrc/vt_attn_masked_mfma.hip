@@ -251,8 +251,14 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
     if (a.window > 0) lo_last = max(lo_last, pos_last - a.window + 1);
 
     // queries as the second operand of v_mfma_f32_16x16x32: a lane holds 8 consecutive elements of its row
+    // (a key size that is no multiple of 32 ends in 16 elements: they take the same instruction with four elements
+    // and four zeros per lane, so that one kind of product feeds an accumulator)
     vt_lowp8_t qf[NK32 > 0 ? NK32 : 1];
-    vt_lowp4_t qtail = {0, 0, 0, 0};
+    auto low_half = [](const bf16_t* p) -> vt_lowp8_t {             // four elements from p, then four zeros
+        const uint2 v = *(const uint2*)p;
+        return __builtin_bit_cast(vt_lowp8_t, make_uint4(v.x, v.y, 0u, 0u));
+    };
+    vt_lowp8_t qtail = __builtin_bit_cast(vt_lowp8_t, make_uint4(0u, 0u, 0u, 0u));
     {
         const bf16_t* qrow = a.q + ((size_t)t * a.H + h) * D;
         const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
@@ -261,7 +267,7 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
             const uint4 raw = row_ok ? *(const uint4*)(qrow + kk * 32 + grp * 8) : zero4;
             qf[kk] = __builtin_bit_cast(vt_lowp8_t, raw);
         }
-        if (TAIL && row_ok) qtail = load4(qrow + (D - 16) + grp * 4);
+        if (TAIL && row_ok) qtail = low_half(qrow + (D - 16) + grp * 4);
     }
     f32x4 acc[NV];
 #pragma unroll
@@ -350,8 +356,8 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
             s1 = VT_MFMA_16X16X32(k1, qf[kk], s1);
         }
         if (TAIL) {
-            s0 = VT_MFMA_16X16X16(load4(kl + (D - 16) + grp * 4), qtail, s0);
-            s1 = VT_MFMA_16X16X16(load4(kl + 16 * KROW + (D - 16) + grp * 4), qtail, s1);
+            s0 = VT_MFMA_16X16X32(low_half(kl + (D - 16) + grp * 4), qtail, s0);
+            s1 = VT_MFMA_16X16X32(low_half(kl + 16 * KROW + (D - 16) + grp * 4), qtail, s1);
         }
         float sc[8];
 #pragma unroll

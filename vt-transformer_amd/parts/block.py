@@ -105,7 +105,8 @@ class HyperBlock(Part):
                  learned_streams: bool = True, token_shift: bool = False, residual_gate: bool = False,
                  names: Optional[Dict[str, str]] = None):
         """names: tensor names behind the layer's prefix, with {} standing for the sublayer's number, for in, out, mix
-        (the streams' numbers), gate and gate_bias (the residual gate's matrix and bias), and for shift (mu)."""
+        (the streams' numbers), gate and gate_bias (the residual gate's matrix and bias), for shift (mu), and for
+        idle_norm (the second norm's tensor of a layer without a feed-forward, where a checkpoint holds one)."""
         self.rt, self.width, self.s = rt, int(width), int(streams)
         if not 1 <= self.s <= ops.STREAMS_MAX:
             raise ValueError(f"{self.s} residual streams (1 to {ops.STREAMS_MAX})")
@@ -116,7 +117,8 @@ class HyperBlock(Part):
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.norm_post = norms["post_mixer"] if feed_forward is not None else None
-        n = {"in": "hc{}.in", "out": "hc{}.out", "mix": "hc{}.mix", "gate": "rg{}", "gate_bias": "rg{}.b", "shift": "shift"}
+        n = {"in": "hc{}.in", "out": "hc{}.out", "mix": "hc{}.mix", "gate": "rg{}", "gate_bias": "rg{}.b", "shift": "shift",
+             "idle_norm": "norm2"}
         n.update(names or {})
         self.names = {k: prefix + v for k, v in n.items()}
         self.n_sub = 1 if feed_forward is None else 2
@@ -142,15 +144,20 @@ class HyperBlock(Part):
         return StateNeed((total,), torch.float32) if total else None
 
     def tensors(self) -> Dict[str, TensorDecl]:
+        """A layer without a feed-forward has no second sublayer; a checkpoint that holds the second sublayer's
+        numbers for it all the same is tolerated, and they are not read."""
         nm, t = self.names, {}
-        for q in range(1, self.n_sub + 1):
+        for q in (1, 2):
+            idle = q > self.n_sub
             if self.learned:
-                t[nm["in"].format(q)] = TensorDecl((self.s,), "gain")
-                t[nm["out"].format(q)] = TensorDecl((self.s,), "gain")
-                t[nm["mix"].format(q)] = TensorDecl((self.s, self.s), "stream_mix")
+                t[nm["in"].format(q)] = TensorDecl((self.s,), "gain", optional=idle)
+                t[nm["out"].format(q)] = TensorDecl((self.s,), "gain", optional=idle)
+                t[nm["mix"].format(q)] = TensorDecl((self.s, self.s), "stream_mix", optional=idle)
             if self.gated:
-                t[nm["gate"].format(q)] = TensorDecl((self.width, self.width), "matrix")
-                t[nm["gate_bias"].format(q)] = TensorDecl((self.width,), "bias")
+                t[nm["gate"].format(q)] = TensorDecl((self.width, self.width), "matrix", optional=idle)
+                t[nm["gate_bias"].format(q)] = TensorDecl((self.width,), "bias", optional=idle)
+        if self.n_sub == 1:
+            t[nm["idle_norm"]] = TensorDecl((self.width,), "gain", optional=True)
         if self.shift:
             t[nm["shift"]] = TensorDecl((self.width,), "bias")
         return t
