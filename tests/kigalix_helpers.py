@@ -129,6 +129,14 @@ def write_model(cfg: dict, folder: str, seed: int, keep_rank: bool = False, idle
     return folder
 
 
+def _row_errors(got: np.ndarray, ref: np.ndarray) -> np.ndarray:
+    """Per row: root mean square of the difference (its mean taken off) over that of the reference (its mean too)."""
+    d = got.astype(np.float64) - ref
+    d = d - d.mean(axis=-1, keepdims=True)
+    c = ref - ref.mean(axis=-1, keepdims=True)
+    return np.sqrt((d * d).mean(axis=-1)) / np.maximum(np.sqrt((c * c).mean(axis=-1)), 1e-30)
+
+
 def check_logits(model_dir: str, reqs: Dict[str, List[int]], steps: List[dict], got: Dict[int, np.ndarray], dtype: str,
                  cache: dict = None) -> float:
     """Every wanted row against the plain implementation's logits at that place; raises at the first row beyond
@@ -136,7 +144,7 @@ def check_logits(model_dir: str, reqs: Dict[str, List[int]], steps: List[dict], 
     cfg, w = pk.read_folder(model_dir)
     cache = cache if cache is not None else {}
     ref = {}
-    close = {}
+    close, limit = {}, {}
     for rid, toks in reqs.items():
         key = (model_dir, tuple(toks))
         if key not in cache:
@@ -144,8 +152,12 @@ def check_logits(model_dir: str, reqs: Dict[str, List[int]], steps: List[dict], 
             logits = pk.forward(cfg, w, toks, margins=margins).numpy()
             least = torch.stack(margins).min(dim=0).values.numpy() if margins else np.full(len(toks), np.inf)
             first = np.nonzero(least < CLOSE_CALL)[0]
-            cache[key] = (logits, int(first[0]) if len(first) else len(toks))
-        ref[rid], close[rid] = cache[key]
+            # what rounding alone does to every position of this model (a model of few channels and many heads, or a
+            # delta layer whose output is divided by a size near zero, moves further than the tolerance): bfloat16 may
+            # differ by three times that where it is more than the tolerance
+            moved = _row_errors(pk.forward(cfg, w, toks, rounded=True).numpy(), logits)
+            cache[key] = (logits, int(first[0]) if len(first) else len(toks), np.maximum(TOL["bfloat16"], 3.0 * moved))
+        ref[rid], close[rid], limit[rid] = cache[key]
     pos = {r: 0 for r in reqs}
     worst, over, count, skipped, far = 0.0, 0, 0, 0, []
     for s in steps:
@@ -160,21 +172,21 @@ def check_logits(model_dir: str, reqs: Dict[str, List[int]], steps: List[dict], 
                 if dtype != "float32" and p >= close[e["id"]]:
                     skipped += 1
                     continue
-                diff = gl - r
-                err = float(np.sqrt(np.mean((diff - diff.mean()) ** 2)) / max(np.sqrt(np.mean((r - r.mean()) ** 2)), 1e-30))
+                err = float(_row_errors(gl[None], r[None])[0])
+                lim = TOL[dtype] if dtype == "float32" else float(limit[e["id"]][p])
                 # float32: every position within the tolerance
                 if dtype == "float32":
                     assert err < TOL[dtype], (f"step {s['step']} request {e['id']} position {p} "
                                               f"(portion starts at {pos[e['id']]}): error {err:.3e} > {TOL[dtype]:.1e}")
-                elif err >= 1.5 * TOL[dtype]:
-                    far.append((s["step"], e["id"], p, pos[e["id"]], round(err, 4)))
-                over += err >= TOL[dtype]
+                elif err >= 1.5 * lim:
+                    far.append((s["step"], e["id"], p, pos[e["id"]], round(err, 4), round(lim, 4)))
+                over += err >= lim
                 count += 1
                 worst = max(worst, err)
             pos[e["id"]] += len(e["tokens"])
     # bfloat16: rounding alone moves a few positions a long way (a delta layer's output is divided by its size, which
     # the first tokens of a sequence can leave near zero), while a lost state, a missed key or a wrong edge moves every
     # position behind it: one position in ten may be over the tolerance, one in forty (or two) half again over it
-    assert over <= max(2, count // 10), f"{over} of {count} positions are over {TOL[dtype]:.0e} (worst {worst:.3e})"
-    assert len(far) <= max(2, count // 40), f"{len(far)} of {count} positions are far over {TOL[dtype]:.0e}: {far[:8]}"
+    assert over <= max(2, count // 10), f"{over} of {count} positions are over their limit (worst {worst:.3e})"
+    assert len(far) <= max(2, count // 40), f"{len(far)} of {count} positions are far over their limit: {far[:8]}"
     return worst

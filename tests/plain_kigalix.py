@@ -156,9 +156,14 @@ def expert_mixture(x: torch.Tensor, w: Dict[str, torch.Tensor], p: str, experts:
 
 
 def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], streams: Optional[list] = None,
-            margins: Optional[list] = None) -> torch.Tensor:
+            margins: Optional[list] = None, rounded: bool = False) -> torch.Tensor:
     """Logits [T, vocab] of one sequence from position 0.  streams: a list that receives the sum of the residual
-    streams after every layer; margins: a list that receives every expert layer's margins (expert_mixture)."""
+    streams after every layer; margins: a list that receives every expert layer's margins (expert_mixture); rounded:
+    every sublayer's input and result and the last norm's output are rounded to bfloat16, which shows how far rounding
+    alone moves this model's logits."""
+    def r16(x):
+        return x.to(torch.bfloat16).to(DT) if rounded else x
+
     w = {k: v.to(DT) for k, v in w.items()}
     eps = float(cfg["norm"]["eps"])
     n_streams = int(cfg.get("streams", 1))
@@ -174,8 +179,8 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], streams: Opti
         else:                                   # one stream and no numbers for it: x <- x + y
             w_in, w_out, w_mix = torch.ones(1, dtype=DT), torch.ones(1, dtype=DT), torch.ones(1, 1, dtype=DT)
         read = sum(w_in[s] * xs[s] for s in range(n_streams))
-        h = offset_rmsnorm(read, w[f"{p}norm{q}"], eps)
-        y = fn(h) * torch.sigmoid(h @ w[f"{p}rg{q}"].T + w[f"{p}rg{q}.b"])
+        h = r16(offset_rmsnorm(read, w[f"{p}norm{q}"], eps))
+        y = r16(r16(fn(h)) * torch.sigmoid(r16(h @ w[f"{p}rg{q}"].T + w[f"{p}rg{q}.b"])))
         xs = [sum(w_mix[s, t] * xs[s] for s in range(n_streams)) + w_out[t] * y for t in range(n_streams)]
 
     for i, layer in enumerate(cfg["layers"]):
@@ -199,7 +204,7 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], streams: Opti
                 raise ValueError(f"feed-forward kind {mlp['kind']!r}")
         if streams is not None:
             streams.append(sum(xs).clone())
-    return offset_rmsnorm(sum(xs), w["final.norm"], eps) @ w["head"].T
+    return r16(offset_rmsnorm(sum(xs), w["final.norm"], eps)) @ w["head"].T
 
 
 def greedy(cfg: dict, w: Dict[str, torch.Tensor], prompt: List[int], n_new: int) -> List[int]:
