@@ -255,6 +255,7 @@ extern "C" int vt_moe_down(const void* act, int dtype, const void* w_down, int w
 #define GR_STAGE ((GR_TB + GR_FB) * GR_LD)
 #define GR_LDS_BYTES (2 * GR_STAGE * 2)
 #define GR_MAX_EXPERTS 1024
+#define GR_FEW_PAIRS 64             // up to so many pairs in a step the products go 16 rows of a matrix to a block
 
 extern "C" int vt_moe_plan_tiles(int pairs, int E) { return (pairs + GR_TB - 1) / GR_TB + E; }
 extern "C" long long vt_moe_plan_size(int pairs, int E) { return 1 + (long long)pairs + 3ll * vt_moe_plan_tiles(pairs, E); }
@@ -474,6 +475,97 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(GroupedArgs a) {
     }
 }
 
+// Few pairs (decoding): an expert's tile holds a handful of pairs, and what bounds the products is how fast the
+// experts' matrices stream in.  A block takes 16 rows of the expert's matrix (gated: 16 gate rows and their up rows)
+// and up to 16 pairs at a time; its four waves split K in turns of 32 and read their operands straight from memory
+// (a lane 16 bytes of its row), four turns' loads in flight; the waves' sums meet in LDS in a fixed order.  Sixteen
+// rows to a block give eight times the blocks of the tiled kernel, which is what fills the GPU when the pairs are few.
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_few_kernel(GroupedArgs a) {
+    const int tile = blockIdx.y;
+    if (tile >= a.plan[0]) return;
+    const int* order = a.plan + 1;
+    const int* tile_expert = order + a.P;
+    const int e = tile_expert[tile], row0 = tile_expert[a.T + tile], rows = tile_expert[2 * a.T + tile];
+    __shared__ float red[3][GATED ? 2 : 1][4][64];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int K = a.K, M = a.M;
+    const int m0 = (int)blockIdx.x * 16;
+    const int mr = min(m0 + r, M - 1);
+    const bf16_t* w0 = a.w + ((size_t)e * (GATED ? 2 : 1) * M + mr) * K;
+    const bf16_t* w1 = GATED ? w0 + (size_t)M * K : w0;
+    const bool scaled = GATED && a.scale;
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    for (int sub = 0; sub < rows; sub += 16) {
+        const int pr = row0 + min(sub + r, rows - 1);       // beyond the tile's pairs the last one again (never stored)
+        const bf16_t* xrow;
+        float xs = 1.f;
+        if (GATED) {
+            const int p = order[pr];
+            xrow = a.x + (size_t)(p / a.top) * K;
+            if (scaled) xs = a.wts[p];
+        } else {
+            xrow = a.x + (size_t)pr * K;
+        }
+        moe_f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+        for (int k0 = 32 * wave; k0 < K; k0 += 128) {
+            const int k = k0 + 8 * g;
+            MoeFrag wa, wb, xf;
+            const bool in = k < K;
+            wa.u = in ? *(const uint4*)(w0 + k) : zero;
+            wb.u = (GATED && in) ? *(const uint4*)(w1 + k) : zero;
+            xf.u = in ? *(const uint4*)(xrow + k) : zero;
+            if (scaled) {
+                xf.u.x = moe_scale2(xf.u.x, xs); xf.u.y = moe_scale2(xf.u.y, xs);
+                xf.u.z = moe_scale2(xf.u.z, xs); xf.u.w = moe_scale2(xf.u.w, xs);
+            }
+            acc0 = VT_MFMA_16X16X32(wa.v, xf.v, acc0);
+            if (GATED) acc1 = VT_MFMA_16X16X32(wb.v, xf.v, acc1);
+        }
+        if (wave) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                red[wave - 1][0][q][lane] = acc0[q];
+                if (GATED) red[wave - 1][GATED ? 1 : 0][q][lane] = acc1[q];
+            }
+        }
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int v = 0; v < 3; ++v)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    acc0[q] += red[v][0][q][lane];
+                    if (GATED) acc1[q] += red[v][GATED ? 1 : 0][q][lane];
+                }
+            // acc[q]: row m0 + 4 g + q of the expert's matrix, pair sub + r of the tile
+            const int row = sub + r, m = m0 + 4 * g;
+            if (row < rows && m < M) {
+                if (GATED) {
+                    float v4[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const float gt = acc0[q], up = acc1[q];
+                        const float z = a.cubic != 0.f ? a.alpha * gt * fmaf(a.cubic * gt, gt, 1.f) : a.alpha * gt;
+                        v4[q] = gt / (1.0f + expf(-z)) * up;
+                    }
+                    uint2 o;
+                    o.x = vt_pack2(v4[0], v4[1]);
+                    o.y = vt_pack2(v4[2], v4[3]);
+                    *(uint2*)((bf16_t*)a.out + (size_t)(row0 + row) * M + m) = o;
+                } else {
+                    const int p = order[row0 + row];
+                    const float s = a.scale ? a.wts[p] : 1.f;
+                    *(float4*)((float*)a.out + (size_t)p * M + m) = make_float4(s * acc0[0], s * acc0[1], s * acc0[2], s * acc0[3]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
 // out[t] = sum of y[t * top + k] over k = 0, 1, .. in that order
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, float* __restrict__ out, int W4, int top,
                                                           long long total4) {
@@ -513,7 +605,8 @@ extern "C" int vt_moe_gate_up_grouped(const void* x, const void* w_gu, const int
     const int P = n * top, T = vt_moe_plan_tiles(P, E);
     VT_REQUIRE(T <= 65535, "vt_moe_gate_up_grouped: too many pairs (%d)", P);
     GroupedArgs a = {(const bf16_t*)x, (const bf16_t*)w_gu, plan, wts, act, P, W, F, top, T, scale_input, alpha, cubic};
-    moe_grouped_kernel<true><<<dim3((F + 63) / 64, T), 256, GR_LDS_BYTES, stream>>>(a);
+    if (P <= GR_FEW_PAIRS) moe_few_kernel<true><<<dim3((F + 15) / 16, T), 256, 0, stream>>>(a);
+    else moe_grouped_kernel<true><<<dim3((F + 63) / 64, T), 256, GR_LDS_BYTES, stream>>>(a);
     VT_CHECK_LAUNCH("vt_moe_gate_up_grouped");
     return 0;
 }
@@ -532,7 +625,8 @@ extern "C" int vt_moe_down_grouped(const void* act, const void* w_down, const in
     VT_REQUIRE(T <= 65535, "vt_moe_down_grouped: too many pairs (%d)", P);
     GroupedArgs a = {(const bf16_t*)act, (const bf16_t*)w_down, plan, wts, top == 1 ? (void*)out : (void*)y, P, F, W, top, T,
                      scale_output, 1.f, 0.f};
-    moe_grouped_kernel<false><<<dim3((W + GR_FB - 1) / GR_FB, T), 256, GR_LDS_BYTES, stream>>>(a);
+    if (P <= GR_FEW_PAIRS) moe_few_kernel<false><<<dim3((W + 15) / 16, T), 256, 0, stream>>>(a);
+    else moe_grouped_kernel<false><<<dim3((W + GR_FB - 1) / GR_FB, T), 256, GR_LDS_BYTES, stream>>>(a);
     VT_CHECK_LAUNCH("vt_moe_down_grouped");
     if (top > 1) {
         const long long total4 = (long long)n * (W / 4);

@@ -53,8 +53,9 @@ class ExpertMixture(Part):
         n.update(names or {})
         self.names = {k: prefix + v for k, v in n.items()}
         self.router = self.w_gu = self.w_down = None
-        # pairs (token, choice) from which the experts' products run grouped on the matrix cores
-        self.grouped_from = 16
+        # pairs (token, choice) from which the experts' products run on the matrix cores, sorted by expert (16-bit types
+        # with sizes in multiples of 8: few pairs 16 rows of a matrix to a block, many in tiles of 128 x 128)
+        self.grouped_from = 1
 
     def tensors(self) -> Dict[str, TensorDecl]:
         nm = self.names
