@@ -477,8 +477,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(GroupedArgs a) {
 
 // Few pairs (decoding): an expert's tile holds a handful of pairs, and what bounds the products is how fast the
 // experts' matrices stream in.  A block takes 16 rows of the expert's matrix (gated: 16 gate rows and their up rows)
-// and up to 16 pairs at a time; its four waves split K in turns of 32 and read their operands straight from memory
-// (a lane 16 bytes of its row), four turns' loads in flight; the waves' sums meet in LDS in a fixed order.  Sixteen
+// and up to 16 pairs at a time; its four waves split K in turns of 64 (a cache line of every row) and read their
+// operands straight from memory (a lane 16 bytes of its row), two turns' loads in flight; the waves' sums meet in LDS in a fixed order.  Sixteen
 // rows to a block give eight times the blocks of the tiled kernel, which is what fills the GPU when the pairs are few.
 template <bool GATED>
 __global__ __launch_bounds__(256) void moe_few_kernel(GroupedArgs a) {
@@ -509,20 +509,27 @@ __global__ __launch_bounds__(256) void moe_few_kernel(GroupedArgs a) {
             xrow = a.x + (size_t)pr * K;
         }
         moe_f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-        for (int k0 = 32 * wave; k0 < K; k0 += 128) {
-            const int k = k0 + 8 * g;
-            MoeFrag wa, wb, xf;
-            const bool in = k < K;
-            wa.u = in ? *(const uint4*)(w0 + k) : zero;
-            wb.u = (GATED && in) ? *(const uint4*)(w1 + k) : zero;
-            xf.u = in ? *(const uint4*)(xrow + k) : zero;
-            if (scaled) {
-                xf.u.x = moe_scale2(xf.u.x, xs); xf.u.y = moe_scale2(xf.u.y, xs);
-                xf.u.z = moe_scale2(xf.u.z, xs); xf.u.w = moe_scale2(xf.u.w, xs);
+        // a wave's turn: 64 of K, one 128-byte line of every row, as two products
+#pragma unroll 2
+        for (int kb = 64 * wave; kb < K; kb += 256) {
+            MoeFrag wa[2], wb[2], xf[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int k = kb + 32 * h + 8 * g;
+                const bool in = k < K;
+                wa[h].u = in ? *(const uint4*)(w0 + k) : zero;
+                wb[h].u = (GATED && in) ? *(const uint4*)(w1 + k) : zero;
+                xf[h].u = in ? *(const uint4*)(xrow + k) : zero;
             }
-            acc0 = VT_MFMA_16X16X32(wa.v, xf.v, acc0);
-            if (GATED) acc1 = VT_MFMA_16X16X32(wb.v, xf.v, acc1);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                if (scaled) {
+                    xf[h].u.x = moe_scale2(xf[h].u.x, xs); xf[h].u.y = moe_scale2(xf[h].u.y, xs);
+                    xf[h].u.z = moe_scale2(xf[h].u.z, xs); xf[h].u.w = moe_scale2(xf[h].u.w, xs);
+                }
+                acc0 = VT_MFMA_16X16X32(wa[h].v, xf[h].v, acc0);
+                if (GATED) acc1 = VT_MFMA_16X16X32(wb[h].v, xf[h].v, acc1);
+            }
         }
         if (wave) {
 #pragma unroll
