@@ -546,7 +546,7 @@ def test_trace_run_with_a_kigalix_folder(folders, tmp_path):
 def random_kigalix_config(seed: int) -> dict:
     rs = np.random.RandomState(seed)
     pick = lambda xs: xs[rs.randint(len(xs))]      # noqa: E731
-    width = int(pick([24, 40, 64, 96, 136]))
+    width = int(pick([24, 40, 52, 64, 96, 100, 136]))       # (52, 100: no multiples of 8)
     layers = []
     for _ in range(rs.randint(2, 6)):
         kind = pick([None, "dense", "moe", "moe"])
