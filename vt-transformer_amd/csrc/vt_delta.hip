@@ -444,18 +444,19 @@ struct GeneralDeltaArgs {
 };
 
 // vt_delta_rule's arrangement: the block's 256 threads are 16 rows of lanes for the recurrence (a row per value
-// column, lane r holding the state elements d = 16 i + r) and TILE tokens x 16 lanes for a tile's inputs, which are
+// column, lane r holding the DS consecutive state elements from d = DS r, so that a token's vectors come out of LDS
+// 16 bytes at a time) and TILE tokens x 16 lanes for a tile's inputs, which are
 // asked for before the recurrence over the tile in front starts.  Per token and column:
 //     p = u . S;   S_d <- w_d S_d - (a_d u_d) p + k_d v;   o = r . S
 // the same instructions in the same order whatever the tile, so nothing depends on how a request was cut.
 template <typename TI, int DS, int TILE>
 __global__ __launch_bounds__(256) void general_delta_kernel(GeneralDeltaArgs a) {
     constexpr int DP = 16 * DS;
-    __shared__ float rs[TILE][DP];      // read-out vectors
-    __shared__ float ks[TILE][DP];      // keys as they come
-    __shared__ float us[TILE][DP];      // unit keys
-    __shared__ float bs[TILE][DP];      // removal rate times unit key
-    __shared__ float ws[TILE][DP];      // decays
+    __shared__ __attribute__((aligned(16))) float rs[TILE][DP];      // read-out vectors
+    __shared__ __attribute__((aligned(16))) float ks[TILE][DP];      // keys as they come
+    __shared__ __attribute__((aligned(16))) float us[TILE][DP];      // unit keys
+    __shared__ __attribute__((aligned(16))) float bs[TILE][DP];      // removal rate times unit key
+    __shared__ __attribute__((aligned(16))) float ws[TILE][DP];      // decays
     __shared__ float vs[TILE][DELTA_GROUPS];
 
     const int e = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * DELTA_GROUPS;
@@ -470,13 +471,13 @@ __global__ __launch_bounds__(256) void general_delta_kernel(GeneralDeltaArgs a) 
     float S[DS];
 #pragma unroll
     for (int i = 0; i < DS; ++i) {
-        const int d = 16 * i + r;
+        const int d = DS * r + i;
         S[i] = (col < Dv && d < D) ? S_head[(size_t)col * D + d] : 0.f;
     }
     float ab[DS];
 #pragma unroll
     for (int i = 0; i < DS; ++i) {
-        const int d = 16 * i + r;
+        const int d = DS * r + i;
         ab[i] = (a.a_bias && d < D) ? a.a_bias[(size_t)h * D + d] : 0.f;
     }
 
@@ -488,7 +489,7 @@ __global__ __launch_bounds__(256) void general_delta_kernel(GeneralDeltaArgs a) 
         const size_t zrow = (size_t)(ok ? t : start) * H * D + (size_t)h * D;
 #pragma unroll
         for (int i = 0; i < DS; ++i) {
-            const int d = 16 * i + r;
+            const int d = DS * r + i;
             const bool in = ok && d < D;
             in_r[i] = in ? load_f32<TI>(x, row + a.r_col + (size_t)h * D + d) : 0.f;
             in_k[i] = in ? load_f32<TI>(x, row + a.k_col + (size_t)h * D + d) : 0.f;
@@ -510,7 +511,7 @@ __global__ __launch_bounds__(256) void general_delta_kernel(GeneralDeltaArgs a) 
             const float rk = 1.0f / sqrtf(sk + a.key_eps);
 #pragma unroll
             for (int i = 0; i < DS; ++i) {
-                const int d = 16 * i + r;
+                const int d = DS * r + i;
                 const float u = in_k[i] * rk;
                 const float rate = 1.0f / (1.0f + expf(-(in_a[i] + ab[i])));
                 rs[cl][d] = in_r[i];
@@ -526,13 +527,13 @@ __global__ __launch_bounds__(256) void general_delta_kernel(GeneralDeltaArgs a) 
         auto token = [&](int tt) {
             float p = 0.f;
 #pragma unroll
-            for (int i = 0; i < DS; ++i) p = fmaf(us[tt][16 * i + r], S[i], p);
+            for (int i = 0; i < DS; ++i) p = fmaf(us[tt][DS * r + i], S[i], p);
             p = row16_sum(p);
             const float v = vs[tt][cl];
             float acc = 0.f;
 #pragma unroll
             for (int i = 0; i < DS; ++i) {
-                const int d = 16 * i + r;
+                const int d = DS * r + i;
                 S[i] = fmaf(ws[tt][d], S[i], fmaf(-bs[tt][d], p, ks[tt][d] * v));
                 acc = fmaf(rs[tt][d], S[i], acc);
             }
@@ -548,7 +549,7 @@ __global__ __launch_bounds__(256) void general_delta_kernel(GeneralDeltaArgs a) 
     }
 #pragma unroll
     for (int i = 0; i < DS; ++i) {
-        const int d = 16 * i + r;
+        const int d = DS * r + i;
         if (col < Dv && d < D) S_head[(size_t)col * D + d] = S[i];
     }
 }
