@@ -59,11 +59,14 @@ class ScheduleEntry:
     entry reads instead of writing its own (None: own cache).
     ``offset_row``: before this entry runs, row ``offset_row`` of the model's
     table of stream offsets (``ModelSpec.stream_offsets``) is added to every
-    token of the residual stream (None: nothing is added)."""
+    token of the residual stream (None: nothing is added).
+    ``inject``: before this entry runs (and before its offset is added), the stream x is replaced by W [x; x0], a
+    projection of the stream joined with the embedding's output x0 (``ModelSpec.stream_inject`` names W)."""
 
     layer: int
     cache_from: Optional[int] = None
     offset_row: Optional[int] = None
+    inject: bool = False
 
 
 @dataclass(frozen=True)
@@ -82,6 +85,9 @@ class ModelSpec:
     # a tensor [rows, hidden_size] of vectors that schedule entries add to the stream before they run
     # (``ScheduleEntry.offset_row``): {"name": tensor name, "rows": number of rows}
     stream_offsets: Optional[Dict[str, Any]] = None
+    # a matrix [hidden_size, 2 * hidden_size] that re-enters the embedding's output into the stream in front of the
+    # schedule entries that say ``inject``: x <- W [x; x0].  {"name": tensor name}
+    stream_inject: Optional[Dict[str, Any]] = None
     # 0: one residual stream [tokens, width].  S >= 1: S copies of it, [tokens, S, width], which all start as the
     # embedding's output and are added up in front of the final norm; the layers' blocks are then of a kind that
     # reads and writes several streams ("hyper")
@@ -91,13 +97,15 @@ class ModelSpec:
         n = len(self.layers)
         if self.streams < 0:
             raise ConfigError(f"{self.streams} residual streams")
-        if self.streams and self.stream_offsets:
+        if self.streams and (self.stream_offsets or self.stream_inject):
             raise ConfigError("stream offsets are added to a single residual stream only")
         for i, e in enumerate(self.schedule):
             if e.offset_row is not None:
                 rows = int(self.stream_offsets["rows"]) if self.stream_offsets else 0
                 if not 0 <= e.offset_row < rows:
                     raise ConfigError(f"schedule[{i}] adds row {e.offset_row} of a table of {rows} stream offsets")
+            if e.inject and not self.stream_inject:
+                raise ConfigError(f"schedule[{i}] re-enters the embedding's output, but the model names no matrix for it")
             if not 0 <= e.layer < n:
                 raise ConfigError(f"schedule[{i}] names layer {e.layer}, model has {n} layers")
             if e.cache_from is not None:

@@ -18,7 +18,14 @@
 //                   value.
 //   vt_qk_prepare also scales the queries of position p by 1 + coef * ln(floor((p + 1) / every) + 1) (every 0: not),
 //                   and mixes values across layers: vmix 1 leaves the token's values in `v_first` (float32), vmix 2
-//                   writes (1 - lambda) v + lambda v_first into the pages instead of v.
+//                   writes (1 - lambda) v + lambda v_first into the pages instead of v.  With `q_gain` / `k_gain`
+//                   ([D], shared by the heads) the unit-RMS queries / keys are multiplied by a gain per element.
+//   vt_attn_masked, further forms of the score and of the weights, each switched on by its pointer or flag:
+//                   `dist_r1`, `dist_r2` ([H] each): r1[head] * ln(1 + r2[head] * (i - j)) is taken off the score;
+//                   `score_shift` ([H]): a number per head is added to every score;
+//                   sigmoid_weights: the weight of a seen key is sigmoid(score) and nothing is normalized (no
+//                   maximum, no sum, no sink); gate_wide: the gate is one logit per output element,
+//                   gate[token][head * Dv + d], instead of one per head.
 #include "vt_common.h"
 #include <math.h>
 
@@ -43,6 +50,8 @@ struct PrepArgs {
     int vmix;               // 0: none; 1: the values go to v_first as well; 2: the pages get (1 - lambda) v + lambda v_first
     float* v_first;         // [n][G * Dv] float32
     const float* v_lambda;  // one float on the device
+    const float* q_gain;    // [D] or null: a gain per element on the unit-RMS queries
+    const float* k_gain;    // [D] or null: likewise for the keys
 };
 
 template <typename TI, typename TC>
@@ -95,6 +104,15 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(PrepArgs a) {
                 r = 1.0f / sqrtf(ss / (float)a.D + a.eps);
             }
             if (is_q && a.q_temp_every > 0) r *= 1.0f + a.q_temp_coef * logf((float)((pos + 1) / a.q_temp_every) + 1.0f);
+            const float* gain = is_q ? a.q_gain : a.k_gain;
+            if (gain) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int d = lane + 64 * i;
+                    if (d < a.D) vals[i] = vals[i] * r * gain[d];
+                }
+                r = 1.f;
+            }
             if (is_q) {
                 TC* dst = (TC*)a.q_out + ((size_t)t * a.H + u) * a.D;
 #pragma unroll
@@ -133,7 +151,7 @@ extern "C" int vt_qk_prepare(const void* x, int x_dtype, long long ldx, const fl
                              int max_blocks, void* q_out, void* k_pages, void* v_pages, int cache_dtype, int page_size,
                              int num_pages, int n, int H, int G, int D, int Dv, int write_kv, int unit_rms, float eps,
                              float q_temp_coef, int q_temp_every, int vmix, float* v_first, const float* v_lambda,
-                             hipStream_t stream) {
+                             const float* q_gain, const float* k_gain, hipStream_t stream) {
     VT_REQUIRE(n >= 0 && H > 0 && G > 0 && H % G == 0, "vt_qk_prepare: bad heads %d/%d", H, G);
     VT_REQUIRE(D > 0 && D <= 256 && Dv > 0, "vt_qk_prepare: head sizes %d/%d (keys up to 256)", D, Dv);
     VT_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= D, "vt_qk_prepare: %d rotated elements of %d", rot, D);
@@ -151,7 +169,7 @@ extern "C" int vt_qk_prepare(const void* x, int x_dtype, long long ldx, const fl
     a.q_out = q_out; a.k_pages = k_pages; a.v_pages = v_pages; a.ldx = ldx; a.H = H; a.G = G; a.D = D; a.Dv = Dv; a.rot = rot;
     a.max_pos = max_pos; a.page_size = page_size; a.max_blocks = max_blocks; a.num_pages = num_pages; a.write_kv = write_kv;
     a.unit_rms = unit_rms; a.eps = eps; a.q_temp_coef = q_temp_coef; a.q_temp_every = q_temp_every; a.vmix = vmix;
-    a.v_first = v_first; a.v_lambda = v_lambda;
+    a.v_first = v_first; a.v_lambda = v_lambda; a.q_gain = q_gain; a.k_gain = k_gain;
     // few tokens: a wave per head, over several blocks per token; many tokens: a block per token goes through its heads
     const int units = H + (write_kv ? 2 * G : 0);
     const dim3 grid(n, n >= 1024 ? 1 : (units + 3) / 4);
@@ -174,8 +192,13 @@ struct MaskedArgs {
     const void* gate;       // gate[t * ldg + h], or null
     const float* sink;      // [H], or null: exp(sink[h]) joins the denominator
     const float* slopes;    // [H], or null: slopes[h] * (position - key index) is taken off every score
+    const float* dist_r1;   // [H] each, or null: r1[h] * ln(1 + r2[h] * (position - key index)) is taken off every score
+    const float* dist_r2;
+    const float* score_shift;   // [H], or null: added to every score
     void* out;              // [n][H][Dv]
     long long ldg;
+    int sigmoid_weights;    // 1: weight = sigmoid(score), not normalized
+    int gate_wide;          // 1: gate[t * ldg + h * Dv + d]
     int H, G, D, Dv, page_size, max_blocks, num_pages, window, chunk;
     float scale, cap;
 };
@@ -200,6 +223,9 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
     const TC* kp = (const TC*)a.k_pages;
     const TC* vp = (const TC*)a.v_pages;
     const float slope = a.slopes ? a.slopes[h] : 0.f;
+    const float r1 = a.dist_r1 ? a.dist_r1[h] : 0.f, r2 = a.dist_r1 ? a.dist_r2[h] : 0.f;
+    const float shift = a.score_shift ? a.score_shift[h] : 0.f;
+    const bool sig = a.sigmoid_weights != 0;
 
     for (int d = tid; d < D; d += KEYS) qs[d] = load_f32<TC>((const TC*)a.q, ((size_t)t * a.H + h) * D + d);
     __syncthreads();
@@ -225,17 +251,26 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
                 s = dot * a.scale;
                 if (a.cap > 0.f) s = a.cap * tanhf(s / a.cap);
                 if (a.slopes) s -= slope * (float)(pos - j);
+                if (a.dist_r1) s -= r1 * log1pf(r2 * (float)(pos - j));
+                s += shift;
             } else {
                 s = __int_as_float(0x7fc00000);  // a missing page must show, not pass as a masked key
             }
         }
-        const float cmax = block_max(s, red);
-        const float m_new = fmaxf(m, cmax);
-        const float p = valid ? expf(s - m_new) : 0.f;
-        sp[tid] = p;
-        const float csum = block_sum(p, red);  // its barriers also publish sp
-        const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
-        l = l * alpha + csum;
+        float m_new = 0.f, alpha = 1.f;
+        if (sig) {
+            // every key's weight stands alone: nothing to rescale
+            sp[tid] = valid ? 1.0f / (1.0f + expf(-s)) : 0.f;
+            __syncthreads();
+        } else {
+            const float cmax = block_max(s, red);
+            m_new = fmaxf(m, cmax);
+            const float p = valid ? expf(s - m_new) : 0.f;
+            sp[tid] = p;
+            const float csum = block_sum(p, red);  // its barriers also publish sp
+            alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
+            l = l * alpha + csum;
+        }
 
         float part = 0.f;
         if (pv_active) {
@@ -275,7 +310,8 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
         __syncthreads();
         m = m_new;
     }
-    if (a.sink) {
+    if (sig) l = 1.f;
+    if (a.sink && !sig) {
         // the sink is one more score with no value behind it
         const float sk = a.sink[h];
         const float m_all = fmaxf(m, sk);
@@ -285,23 +321,18 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
 #pragma unroll
         for (int c = 0; c < 3; ++c) acc_w[c] *= keep;
     }
-    float f = 1.0f / l;
-    if (a.gate) {
-        const float z = load_f32<TG>((const TG*)a.gate, (size_t)t * a.ldg + h);
-        f = (1.0f / (1.0f + expf(-z))) / l;
-    }
-    if (tid < Dv) {
-        float o = acc / l;
-        if (a.gate) {
-            const float z = load_f32<TG>((const TG*)a.gate, (size_t)t * a.ldg + h);
-            o *= 1.0f / (1.0f + expf(-z));
-        }
-        store_f32<TC>((TC*)a.out, ((size_t)t * a.H + h) * Dv + tid, o);
-    }
+    // the gate's logit of output element d: one per head, or one per element
+    auto gate_of = [&](int d) -> float {
+        if (!a.gate) return 1.f;
+        const float z = load_f32<TG>((const TG*)a.gate, (size_t)t * a.ldg + (a.gate_wide ? (size_t)h * Dv + d : (size_t)h));
+        return 1.0f / (1.0f + expf(-z));
+    };
+    if (tid < Dv) store_f32<TC>((TC*)a.out, ((size_t)t * a.H + h) * Dv + tid, (acc / l) * gate_of(tid));
     if (wide) {
 #pragma unroll
         for (int c = 1; c < 4; ++c)
-            if (tid + c * KEYS < Dv) store_f32<TC>((TC*)a.out, ((size_t)t * a.H + h) * Dv + tid + c * KEYS, acc_w[c - 1] * f);
+            if (tid + c * KEYS < Dv)
+                store_f32<TC>((TC*)a.out, ((size_t)t * a.H + h) * Dv + tid + c * KEYS, acc_w[c - 1] * (gate_of(tid + c * KEYS) / l));
     }
 }
 
@@ -309,8 +340,12 @@ extern "C" int vt_attn_masked(const void* q, const void* k_pages, const void* v_
                               const int* tok_entry, const int* block_table, const void* gate, int gate_dtype,
                               long long ldg, void* out, int n, int H, int G, int D, int Dv, int page_size,
                               int max_blocks, int num_pages, int window, int chunk, float scale, float cap,
-                              const float* sink, const float* slopes, hipStream_t stream) {
+                              const float* sink, const float* slopes, const float* dist_r1, const float* dist_r2,
+                              const float* score_shift, int sigmoid_weights, int gate_wide, hipStream_t stream) {
     VT_REQUIRE(n >= 0 && H > 0 && G > 0 && H % G == 0, "vt_attn_masked: bad heads %d/%d", H, G);
+    VT_REQUIRE((dist_r1 == nullptr) == (dist_r2 == nullptr), "vt_attn_masked: the distance bias takes both of its numbers");
+    VT_REQUIRE(!(sigmoid_weights && sink), "vt_attn_masked: sigmoid weights have no denominator for a sink to join");
+    VT_REQUIRE(!gate_wide || ldg >= (long long)H * Dv, "vt_attn_masked: gate rows are too short");
     VT_REQUIRE(D > 0 && D <= 8192 && Dv > 0 && Dv <= 4 * KEYS, "vt_attn_masked: head sizes %d/%d (keys up to 8192, values up to %d)", D, Dv, 4 * KEYS);
     VT_REQUIRE(page_size > 0 && max_blocks > 0 && num_pages > 0, "vt_attn_masked: bad cache sizes");
     VT_REQUIRE(H <= 65535, "vt_attn_masked: too many heads (%d)", H);
@@ -320,7 +355,8 @@ extern "C" int vt_attn_masked(const void* q, const void* k_pages, const void* v_
     a.q = q; a.k_pages = k_pages; a.v_pages = v_pages; a.positions = positions; a.tok_entry = tok_entry;
     a.block_table = block_table; a.gate = gate; a.out = out; a.ldg = ldg; a.H = H; a.G = G; a.D = D; a.Dv = Dv;
     a.page_size = page_size; a.max_blocks = max_blocks; a.num_pages = num_pages; a.window = window; a.chunk = chunk;
-    a.scale = scale; a.cap = cap; a.sink = sink; a.slopes = slopes;
+    a.scale = scale; a.cap = cap; a.sink = sink; a.slopes = slopes; a.dist_r1 = dist_r1; a.dist_r2 = dist_r2;
+    a.score_shift = score_shift; a.sigmoid_weights = sigmoid_weights; a.gate_wide = gate_wide;
     const size_t shmem = (size_t)(D + 2 * KEYS) * sizeof(float);
     const dim3 grid(n, H);
     if (dtype == VT_F32) {

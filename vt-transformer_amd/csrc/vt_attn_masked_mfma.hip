@@ -12,7 +12,11 @@
 //                      its value element), B = P^T, which is exactly what the lane holds of S^T
 // so the probabilities never leave the registers.  Scores, softmax and sums are float32.
 // With `slopes`, slopes[head] * (position - key index) is taken off every score; with `sink`, exp(sink[head]) joins
-// the softmax's denominator (a key that holds no value).
+// the softmax's denominator (a key that holds no value).  Further forms, each switched on by its pointer or flag:
+// `dist_r1`, `dist_r2`: r1[head] * ln(1 + r2[head] * (position - key index)) is taken off every score (base 2:
+// r1 * log2(1 + r2 d), the hardware's logarithm); `score_shift`: a number per head added to every score;
+// sigmoid_weights: the weight of a seen key is sigmoid(score) = 1 / (1 + 2^-score'), nothing is normalized;
+// gate_wide: one gate logit per output element, gate[token][head * Dv + d], instead of one per head.
 #include "vt_common.h"
 #include <math.h>
 
@@ -37,11 +41,43 @@ struct MfmaArgs {
     const void* gate;       // gate[t * ldg + h], or null
     const float* sink;      // [H] or null
     const float* slopes;    // [H] or null
+    const float* dist_r1;   // [H] each, or null
+    const float* dist_r2;
+    const float* score_shift;   // [H] or null
     bf16_t* out;            // [n][H][Dv]
     long long ldg;
-    int n_tiles, H, G, page_size, max_blocks, num_pages, window, chunk, gate_f32;
+    int n_tiles, H, G, page_size, max_blocks, num_pages, window, chunk, gate_f32, sigmoid_weights, gate_wide;
     float scale, cap;
 };
+
+// what the score's optional forms take off or add, in the base-2 domain: key j seen from position pos
+struct ScoreForms {
+    float slope2, r1, r2, shift2;
+    bool has_slope, has_log;
+    __device__ __forceinline__ float apply(float sc, int pos, int j) const {
+        const float dist = (float)max(pos - j, 0);
+        if (has_slope) sc -= slope2 * dist;
+        if (has_log) sc -= r1 * __builtin_amdgcn_logf(fmaf(r2, dist, 1.0f));
+        return sc + shift2;
+    }
+};
+__device__ __forceinline__ ScoreForms score_forms(const float* slopes, const float* r1, const float* r2, const float* shift, int h) {
+    const float LOG2E = 1.4426950408889634f;
+    ScoreForms f;
+    f.has_slope = slopes != nullptr;
+    f.has_log = r1 != nullptr;
+    f.slope2 = slopes ? slopes[h] * LOG2E : 0.f;
+    f.r1 = r1 ? r1[h] : 0.f;          // r1 ln(x) log2(e) = r1 log2(x)
+    f.r2 = r1 ? r2[h] : 0.f;
+    f.shift2 = shift ? shift[h] * LOG2E : 0.f;
+    return f;
+}
+// the gate on output element d of head h of token t
+__device__ __forceinline__ float gate_at(const void* gate, int gate_f32, long long ldg, int t, size_t column) {
+    const size_t gi = (size_t)t * ldg + column;
+    const float z = gate_f32 ? ((const float*)gate)[gi] : bf16_to_f32(((const bf16_t*)gate)[gi]);
+    return 1.0f / (1.0f + expf(-z));
+}
 
 __device__ __forceinline__ vt_lowp4_t load4(const bf16_t* p) { return *(const vt_lowp4_t*)p; }
 
@@ -86,7 +122,9 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
     const float LOG2E = 1.4426950408889634f;
     const float c1 = a.cap > 0.f ? a.scale * 2.0f * LOG2E / a.cap : a.scale * LOG2E;
     const float c2 = a.cap * LOG2E;
-    const float slope2 = a.slopes ? a.slopes[h] * LOG2E : 0.f;
+    const ScoreForms forms = score_forms(a.slopes, a.dist_r1, a.dist_r2, a.score_shift, h);
+    const bool forms_on = a.slopes || a.dist_r1 || a.score_shift;
+    const bool sig = a.sigmoid_weights != 0;
     const int lo_last = [&] {
         int v = a.chunk > 0 ? (pos_last / a.chunk) * a.chunk : 0;
         if (a.window > 0) v = max(v, pos_last - a.window + 1);
@@ -148,9 +186,9 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
                 sc[i] = x;
             }
         }
-        if (a.slopes) {
+        if (forms_on) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) sc[i] -= slope2 * (float)(pos - (kt + (i < 4 ? 0 : 16) + grp * 4 + (i & 3)));
+            for (int i = 0; i < 8; ++i) sc[i] = forms.apply(sc[i], pos, kt + (i < 4 ? 0 : 16) + grp * 4 + (i & 3));
         }
         // a turn that every row sees whole needs no mask
         const bool whole = kt + 31 <= pos_first && kt >= lo_last && ok_now[0] && ok_now[1];
@@ -163,20 +201,27 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
                 sc[i] = seen ? (ok_now[i >> 2] ? sc[i] : nan) : -INFINITY;
             }
         }
-        float mt = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-        const float m_new = fmaxf(m, mt);
-        const float mref = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
-        float p[8], psum = 0.f;
+        float p[8], alpha = 1.f;
+        if (sig) {
+            // every key's weight stands alone: 1 / (1 + 2^-s), and 0 for a masked key (s = -inf)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            p[i] = __builtin_amdgcn_exp2f(sc[i] - mref);
-            psum += p[i];
+            for (int i = 0; i < 8; ++i) p[i] = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-sc[i]));
+        } else {
+            float mt = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+            mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float m_new = fmaxf(m, mt);
+            const float mref = (m_new == -INFINITY) ? 0.f : m_new;
+            alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                p[i] = __builtin_amdgcn_exp2f(sc[i] - mref);
+                psum += p[i];
+            }
+            l = l * alpha + psum;
+            m = m_new;
         }
-        l = l * alpha + psum;
-        m = m_new;
         struct U2 { unsigned a, b; };
         const U2 pk0 = {vt_pack2(p[0], p[1]), vt_pack2(p[2], p[3])}, pk1 = {vt_pack2(p[4], p[5]), vt_pack2(p[6], p[7])};
         const vt_lowp4_t pf0 = __builtin_bit_cast(vt_lowp4_t, pk0), pf1 = __builtin_bit_cast(vt_lowp4_t, pk1);
@@ -190,7 +235,7 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (!row_ok) return;
-    if (a.sink) {
+    if (a.sink && !sig) {
         // the sink is one more score with no value behind it (scores are kept times log2 e)
         const float sk = a.sink[h] * LOG2E;
         const float m_all = fmaxf(m, sk);
@@ -199,17 +244,17 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) acc[v] *= keep;
     }
-    float gate = 1.f;
-    if (a.gate) {
-        const size_t gi = (size_t)t * a.ldg + h;
-        const float z = a.gate_f32 ? ((const float*)a.gate)[gi] : bf16_to_f32(((const bf16_t*)a.gate)[gi]);
-        gate = 1.0f / (1.0f + expf(-z));
-    }
-    const float f = gate / l;
+    if (sig) l = 1.f;
+    const float f = ((a.gate && !a.gate_wide) ? gate_at(a.gate, a.gate_f32, a.ldg, t, h) : 1.f) / l;
     bf16_t* o = a.out + ((size_t)t * a.H + h) * DV + grp * 4;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        struct { unsigned a, b; } ok = {vt_pack2(acc[v][0] * f, acc[v][1] * f), vt_pack2(acc[v][2] * f, acc[v][3] * f)};
+        float g4[4] = {f, f, f, f};
+        if (a.gate && a.gate_wide) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) g4[i] = f * gate_at(a.gate, a.gate_f32, a.ldg, t, (size_t)h * DV + v * 16 + grp * 4 + i);
+        }
+        struct { unsigned a, b; } ok = {vt_pack2(acc[v][0] * g4[0], acc[v][1] * g4[1]), vt_pack2(acc[v][2] * g4[2], acc[v][3] * g4[3])};
         *(uint2*)(o + v * 16) = __builtin_bit_cast(uint2, ok);
     }
 }
@@ -277,7 +322,9 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
     const float LOG2E = 1.4426950408889634f;
     const float c1 = a.cap > 0.f ? a.scale * 2.0f * LOG2E / a.cap : a.scale * LOG2E;
     const float c2 = a.cap * LOG2E;
-    const float slope2 = a.slopes ? a.slopes[h] * LOG2E : 0.f;
+    const ScoreForms forms = score_forms(a.slopes, a.dist_r1, a.dist_r2, a.score_shift, h);
+    const bool forms_on = a.slopes || a.dist_r1 || a.score_shift;
+    const bool sig = a.sigmoid_weights != 0;
 
     auto page_of = [&](int kt) -> int {
         const int blk = kt / ps;
@@ -370,9 +417,9 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
                 sc[i] = x;
             }
         }
-        if (a.slopes) {
+        if (forms_on) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) sc[i] -= slope2 * (float)(pos - (kt + (i < 4 ? 0 : 16) + grp * 4 + (i & 3)));
+            for (int i = 0; i < 8; ++i) sc[i] = forms.apply(sc[i], pos, kt + (i < 4 ? 0 : 16) + grp * 4 + (i & 3));
         }
         const bool whole = kt + 31 <= pos_first && kt >= lo_last && ok_now[0] && ok_now[1];
         if (!whole) {
@@ -383,20 +430,27 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
                 sc[i] = seen ? (ok_now[i >> 2] ? sc[i] : nan) : -INFINITY;
             }
         }
-        float mt = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-        const float m_new = fmaxf(m, mt);
-        const float mref = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
-        float p[8], psum = 0.f;
+        float p[8], alpha = 1.f;
+        if (sig) {
+            // every key's weight stands alone: 1 / (1 + 2^-s), and 0 for a masked key (s = -inf)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            p[i] = __builtin_amdgcn_exp2f(sc[i] - mref);
-            psum += p[i];
+            for (int i = 0; i < 8; ++i) p[i] = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-sc[i]));
+        } else {
+            float mt = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+            mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float m_new = fmaxf(m, mt);
+            const float mref = (m_new == -INFINITY) ? 0.f : m_new;
+            alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                p[i] = __builtin_amdgcn_exp2f(sc[i] - mref);
+                psum += p[i];
+            }
+            l = l * alpha + psum;
+            m = m_new;
         }
-        l = l * alpha + psum;
-        m = m_new;
         // One product over the turn's 32 keys.  Its key index 8 grp + j stands for key 4 grp + j of the first run
         // (j < 4) and key 16 + 4 grp + j - 4 of the second: that is the order of the lane's eight probabilities, and the
         // values are read from LDS in the same order.
@@ -415,7 +469,7 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (!row_ok) return;
-    if (a.sink) {
+    if (a.sink && !sig) {
         // the sink is one more score with no value behind it (scores are kept times log2 e)
         const float sk = a.sink[h] * LOG2E;
         const float m_all = fmaxf(m, sk);
@@ -424,17 +478,17 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
 #pragma unroll
         for (int v = 0; v < NV; ++v) acc[v] *= keep;
     }
-    float gate = 1.f;
-    if (a.gate) {
-        const size_t gi = (size_t)t * a.ldg + h;
-        const float z = a.gate_f32 ? ((const float*)a.gate)[gi] : bf16_to_f32(((const bf16_t*)a.gate)[gi]);
-        gate = 1.0f / (1.0f + expf(-z));
-    }
-    const float f = gate / l;
+    if (sig) l = 1.f;
+    const float f = ((a.gate && !a.gate_wide) ? gate_at(a.gate, a.gate_f32, a.ldg, t, h) : 1.f) / l;
     bf16_t* o = a.out + ((size_t)t * a.H + h) * DV + grp * 4;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        struct { unsigned a, b; } ok = {vt_pack2(acc[v][0] * f, acc[v][1] * f), vt_pack2(acc[v][2] * f, acc[v][3] * f)};
+        float g4[4] = {f, f, f, f};
+        if (a.gate && a.gate_wide) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) g4[i] = f * gate_at(a.gate, a.gate_f32, a.ldg, t, (size_t)h * DV + v * 16 + grp * 4 + i);
+        }
+        struct { unsigned a, b; } ok = {vt_pack2(acc[v][0] * g4[0], acc[v][1] * g4[1]), vt_pack2(acc[v][2] * g4[2], acc[v][3] * g4[3])};
         *(uint2*)(o + v * 16) = __builtin_bit_cast(uint2, ok);
     }
 }
@@ -458,11 +512,14 @@ struct DecodeArgs {
     const int* block_table;
     const float* sink;
     const float* slopes;
+    const float* dist_r1;
+    const float* dist_r2;
+    const float* score_shift;
     const void* gate;
     float* part;
     bf16_t* out;            // [n][H][DV]
     long long ldg;
-    int n, H, G, HT, P, page_size, max_blocks, num_pages, window, chunk, gate_f32;
+    int n, H, G, HT, P, page_size, max_blocks, num_pages, window, chunk, gate_f32, sigmoid_weights, gate_wide;
     float scale, cap;
 };
 #define DEC_ROW (VT_VALUE_DIM + 4)
@@ -502,7 +559,9 @@ __global__ __launch_bounds__(256) void attn_masked_decode_kernel(DecodeArgs a) {
     const float LOG2E = 1.4426950408889634f;
     const float c1 = a.cap > 0.f ? a.scale * 2.0f * LOG2E / a.cap : a.scale * LOG2E;
     const float c2 = a.cap * LOG2E;
-    const float slope2 = a.slopes ? a.slopes[h] * LOG2E : 0.f;
+    const ScoreForms forms = score_forms(a.slopes, a.dist_r1, a.dist_r2, a.score_shift, h);
+    const bool forms_on = a.slopes || a.dist_r1 || a.score_shift;
+    const bool sig = a.sigmoid_weights != 0;
 
     for (int turn = p; turn < turns; turn += a.P) {
         const int kt = kt0 + turn * 32;
@@ -540,25 +599,33 @@ __global__ __launch_bounds__(256) void attn_masked_decode_kernel(DecodeArgs a) {
                 sc[i] = x;
             }
             const int j = kt + (i < 4 ? 0 : 16) + grp * 4 + (i & 3);
-            if (a.slopes) sc[i] -= slope2 * (float)(pos - j);
+            if (forms_on) sc[i] = forms.apply(sc[i], pos, j);
             const bool seen = row_ok && j <= pos && j >= lo;
             // (a missing page must show, not pass as a masked key)
             sc[i] = seen ? (ok[i >> 2] ? sc[i] : nan) : -INFINITY;
         }
-        float mt = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-        const float m_new = fmaxf(m, mt);
-        const float mref = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
-        float pr[8], psum = 0.f;
+        float pr[8], alpha = 1.f;
+        if (sig) {
+            // weights that stand alone: the part's "maximum" is 0 so that the merge adds the parts as they are
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            pr[i] = __builtin_amdgcn_exp2f(sc[i] - mref);
-            psum += pr[i];
+            for (int i = 0; i < 8; ++i) pr[i] = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-sc[i]));
+            m = 0.f;
+        } else {
+            float mt = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+            mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float m_new = fmaxf(m, mt);
+            const float mref = (m_new == -INFINITY) ? 0.f : m_new;
+            alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                pr[i] = __builtin_amdgcn_exp2f(sc[i] - mref);
+                psum += pr[i];
+            }
+            l = l * alpha + psum;
+            m = m_new;
         }
-        l = l * alpha + psum;
-        m = m_new;
         struct U2 { unsigned a, b; };
         const U2 pk0 = {vt_pack2(pr[0], pr[1]), vt_pack2(pr[2], pr[3])}, pk1 = {vt_pack2(pr[4], pr[5]), vt_pack2(pr[6], pr[7])};
         const vt_lowp4_t pf0 = __builtin_bit_cast(vt_lowp4_t, pk0), pf1 = __builtin_bit_cast(vt_lowp4_t, pk1);
@@ -604,7 +671,7 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void attn_masked_decode_merge_ker
     }
     float m_all = wave_max(mp);
     float extra = 0.f;
-    if (a.sink) {
+    if (a.sink && !a.sigmoid_weights) {
         // the sink is one more score with no value behind it
         const float sk = a.sink[h] * LOG2E;
         const float top = fmaxf(m_all, sk);
@@ -612,23 +679,19 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void attn_masked_decode_merge_ker
         m_all = top;
     }
     const float w = mp == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mp - m_all);
-    const float l = wave_sum(lp * w) + extra;
+    float l = wave_sum(lp * w) + extra;
+    if (a.sigmoid_weights) l = 1.f;             // (the parts' maxima are all 0 or none: every weight is 1)
     ws[lane] = w;
     wave_lds_order();
-    float gate = 1.f;
-    if (a.gate) {
-        const size_t gi = (size_t)t * a.ldg + h;
-        const float z = a.gate_f32 ? ((const float*)a.gate)[gi] : bf16_to_f32(((const bf16_t*)a.gate)[gi]);
-        gate = 1.0f / (1.0f + expf(-z));
-    }
-    const float f = gate / l;
+    const float f = ((a.gate && !a.gate_wide) ? gate_at(a.gate, a.gate_f32, a.ldg, t, h) : 1.f) / l;
     bf16_t* o = a.out + ((size_t)t * a.H + h) * DV;
     const int d = threadIdx.x;                  // a wave per 64 value elements
     if (d < DV) {
         float sum = 0.f;
 #pragma unroll 8
         for (int p = 0; p < a.P; ++p) sum = fmaf(base[p * step + d], ws[p], sum);
-        o[d] = f32_to_bf16(sum * f);
+        const float g = (a.gate && a.gate_wide) ? gate_at(a.gate, a.gate_f32, a.ldg, t, (size_t)h * DV + d) : 1.f;
+        o[d] = f32_to_bf16(sum * f * g);
     }
 }
 
@@ -637,7 +700,11 @@ extern "C" int vt_attn_masked_decode(const void* q, const void* k_pages, const v
                                      long long ldg, void* out, float* part, long long part_floats, int splits, int n,
                                      int H, int G, int D, int Dv, int page_size, int max_blocks, int num_pages, int window,
                                      int chunk, float scale, float cap, const float* sink, const float* slopes,
-                                     hipStream_t stream) {
+                                     const float* dist_r1, const float* dist_r2, const float* score_shift,
+                                     int sigmoid_weights, int gate_wide, hipStream_t stream) {
+    VT_REQUIRE((dist_r1 == nullptr) == (dist_r2 == nullptr), "vt_attn_masked_decode: the distance bias takes both of its numbers");
+    VT_REQUIRE(!(sigmoid_weights && sink), "vt_attn_masked_decode: sigmoid weights have no denominator for a sink to join");
+    VT_REQUIRE(!gate_wide || !gate || ldg >= (long long)H * Dv, "vt_attn_masked_decode: gate rows are too short");
     VT_REQUIRE(D == VT_KEY_DIM && Dv == VT_VALUE_DIM, "vt_attn_masked_decode: built for heads of %d/%d, called with %d/%d",
                VT_KEY_DIM, VT_VALUE_DIM, D, Dv);
     VT_REQUIRE(n >= 0 && H > 0 && G > 0 && H % G == 0, "vt_attn_masked_decode: bad heads %d/%d", H, G);
@@ -657,7 +724,8 @@ extern "C" int vt_attn_masked_decode(const void* q, const void* k_pages, const v
     a.tok_entry = tok_entry; a.block_table = block_table; a.sink = sink; a.slopes = slopes; a.gate = gate; a.part = part;
     a.out = (bf16_t*)out; a.ldg = ldg; a.n = n; a.H = H; a.G = G; a.HT = HT; a.P = 4 * splits; a.page_size = page_size;
     a.max_blocks = max_blocks; a.num_pages = num_pages; a.window = window; a.chunk = chunk; a.gate_f32 = gate_dtype == VT_F32;
-    a.scale = scale; a.cap = cap;
+    a.scale = scale; a.cap = cap; a.dist_r1 = dist_r1; a.dist_r2 = dist_r2; a.score_shift = score_shift;
+    a.sigmoid_weights = sigmoid_weights; a.gate_wide = gate_wide;
     attn_masked_decode_kernel<<<dim3(splits, G * HT, n), 256, 0, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_masked_decode");
     attn_masked_decode_merge_kernel<<<dim3(H, n), 64 * MERGE_WAVES, 0, stream>>>(a);
@@ -679,7 +747,12 @@ extern "C" int vt_attn_masked_mfma(const void* q, const void* k_pages, const voi
                                    const int* tok_entry, const int* block_table, const int* tiles, int n_tiles,
                                    const void* gate, int gate_dtype, long long ldg, void* out, int H, int G, int D, int Dv,
                                    int page_size, int max_blocks, int num_pages, int window, int chunk, float scale,
-                                   float cap, const float* sink, const float* slopes, hipStream_t stream) {
+                                   float cap, const float* sink, const float* slopes, const float* dist_r1,
+                                   const float* dist_r2, const float* score_shift, int sigmoid_weights, int gate_wide,
+                                   hipStream_t stream) {
+    VT_REQUIRE((dist_r1 == nullptr) == (dist_r2 == nullptr), "vt_attn_masked_mfma: the distance bias takes both of its numbers");
+    VT_REQUIRE(!(sigmoid_weights && sink), "vt_attn_masked_mfma: sigmoid weights have no denominator for a sink to join");
+    VT_REQUIRE(!gate_wide || !gate || ldg >= (long long)H * Dv, "vt_attn_masked_mfma: gate rows are too short");
     VT_REQUIRE(D == VT_KEY_DIM && Dv == VT_VALUE_DIM, "vt_attn_masked_mfma: built for heads of %d/%d, called with %d/%d",
                VT_KEY_DIM, VT_VALUE_DIM, D, Dv);
     VT_REQUIRE(n_tiles >= 0 && H > 0 && G > 0 && H % G == 0, "vt_attn_masked_mfma: bad heads %d/%d", H, G);
@@ -693,7 +766,8 @@ extern "C" int vt_attn_masked_mfma(const void* q, const void* k_pages, const voi
     a.tok_entry = tok_entry; a.block_table = block_table; a.tiles = tiles; a.gate = gate; a.out = (bf16_t*)out; a.ldg = ldg;
     a.n_tiles = n_tiles; a.H = H; a.G = G; a.page_size = page_size; a.max_blocks = max_blocks; a.num_pages = num_pages;
     a.window = window; a.chunk = chunk; a.gate_f32 = gate_dtype == VT_F32; a.scale = scale; a.cap = cap;
-    a.sink = sink; a.slopes = slopes;
+    a.sink = sink; a.slopes = slopes; a.dist_r1 = dist_r1; a.dist_r2 = dist_r2; a.score_shift = score_shift;
+    a.sigmoid_weights = sigmoid_weights; a.gate_wide = gate_wide;
     const long long items = (long long)n_tiles * H;
     if ((H / G) % 4 == 0)       // four heads of one key/value group to a block: they share what they read
         attn_masked_mfma_shared_kernel<<<(unsigned)(items / 4), 256, 0, stream>>>(a);

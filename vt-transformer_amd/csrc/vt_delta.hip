@@ -21,8 +21,21 @@
 // the state lies along the unit key, scaled per channel:
 //     S <- diag(w) S - (a * u)(u^T S) + k v^T,  u = k / sqrt(|k|^2 + eps);   o = S^T r      (both terms read the old S)
 // with w = exp(-c * sigmoid(z)) from decay logits z and a = sigmoid(removal logits), all in float32.
-//   vt_lowrank_tanh:      z[t][j] = bias[j] + sum_l W2[j][l] tanh(x[t][l]): the decay logits from a low-rank projection.
+//   vt_lowrank_tanh:      z[t][j] = bias[j] + sum_l W2[j][l] tanh(x[t][l]): the decay logits from a low-rank projection
+//                         (act 0: without the tanh, for low-rank projections whose middle is linear).
 //   vt_general_delta:     the recurrence, in vt_delta_rule's arrangement (a row of 16 lanes per state column).
+//
+// The gated delta rule with a decay per key channel (vt_delta_rule_channel): the first rule above with
+//     S <- diag(g) S,   g[d] = exp(-exp(A_log[head]) softplus(z[d]))
+// from decay logits z [n][H * D] in float32 (their bias already added).
+//
+// The matrix memory of xLSTM (vt_matrix_memory): per head S [D][Dv], a normalizer n [D] and a running maximum m of
+// the gates' logarithms, all float32 and all zero at the start of a sequence:
+//     i = cap tanh(a_i / cap),  f = logsigmoid(cap tanh(a_f / cap))           from the gates' logits a_i, a_f
+//     m' = max(f + m, i);  S <- e^(f + m - m') S + e^(i - m') k v^T;  n <- e^(f + m - m') n + e^(i - m') k
+//     o = S^T q / (max(|n . q|, e^(-m')) + 1e-6)
+// in vt_delta_rule's arrangement; every block of 16 value columns carries n and m for itself (they are kept once
+// per block of columns in the state, so that no block reads what another has already moved on).
 #include "vt_common.h"
 #include <math.h>
 
@@ -397,10 +410,14 @@ extern "C" int vt_gated_rmsnorm(const float* o, const float* w, const void* gate
 // z[t][j] = bias[j] + sum_l W2[j][l] * tanh(x[t * ldx + l]), l = 0, 1, .. in that order, float32
 template <typename TI, typename TW>
 __global__ __launch_bounds__(256) void lowrank_tanh_kernel(const TI* __restrict__ x, long long ldx, const TW* __restrict__ w2,
-                                                           const float* __restrict__ bias, float* __restrict__ z, int L, int M) {
+                                                           const float* __restrict__ bias, float* __restrict__ z, int L, int M,
+                                                           int act) {
     extern __shared__ float th[];
     const int t = blockIdx.x;
-    for (int l = threadIdx.x; l < L; l += 256) th[l] = tanhf(load_f32<TI>(x, (size_t)t * ldx + l));
+    for (int l = threadIdx.x; l < L; l += 256) {
+        const float v = load_f32<TI>(x, (size_t)t * ldx + l);
+        th[l] = act ? tanhf(v) : v;
+    }
     __syncthreads();
     const int j = blockIdx.y * 256 + threadIdx.x;
     if (j >= M) return;
@@ -410,18 +427,19 @@ __global__ __launch_bounds__(256) void lowrank_tanh_kernel(const TI* __restrict_
 }
 
 extern "C" int vt_lowrank_tanh(const void* x, int x_dtype, long long ldx, const void* w2, int w_dtype, const float* bias,
-                               float* z, int n, int L, int M, hipStream_t stream) {
+                               float* z, int n, int L, int M, int act, hipStream_t stream) {
     VT_REQUIRE(n >= 0 && L > 0 && L <= 8192 && M > 0 && ldx >= L, "vt_lowrank_tanh: bad sizes n=%d L=%d M=%d", n, L, M);
+    VT_REQUIRE(act == 0 || act == 1, "vt_lowrank_tanh: act %d (0: none, 1: tanh)", act);
     VT_REQUIRE(M <= 65535 * 256, "vt_lowrank_tanh: too many outputs");
     if (n == 0) return 0;
     const dim3 grid(n, (M + 255) / 256);
     const size_t lds = (size_t)L * sizeof(float);
     if (x_dtype == VT_F32 && w_dtype == VT_F32)
-        lowrank_tanh_kernel<float, float><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const float*)w2, bias, z, L, M);
+        lowrank_tanh_kernel<float, float><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const float*)w2, bias, z, L, M, act);
     else if (x_dtype == VT_F32 && w_dtype == VT_BF16)
-        lowrank_tanh_kernel<float, bf16_t><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const bf16_t*)w2, bias, z, L, M);
+        lowrank_tanh_kernel<float, bf16_t><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const bf16_t*)w2, bias, z, L, M, act);
     else if (x_dtype == VT_BF16 && w_dtype == VT_BF16)
-        lowrank_tanh_kernel<bf16_t, bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w2, bias, z, L, M);
+        lowrank_tanh_kernel<bf16_t, bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w2, bias, z, L, M, act);
     else return vt_fail("vt_lowrank_tanh: dtypes %d / %d are not handled", x_dtype, w_dtype);
     VT_CHECK_LAUNCH("vt_lowrank_tanh");
     return 0;
@@ -584,5 +602,330 @@ extern "C" int vt_general_delta(const void* x, int dtype, long long ldx, int r_c
     else return vt_fail("vt_general_delta: unknown dtype %d", dtype);
 #undef VT_GDELTA
     VT_CHECK_LAUNCH("vt_general_delta");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+struct ChannelDeltaArgs {
+    const void* qkv;        // [n][C]: q (G x D), k (G x D), v (H x Dv), after convolution and SiLU
+    const void* beta;       // beta[t * ldb + h]: logits of the write strength
+    const float* z;         // [n][H * D] decay logits, float32
+    const float* a_log;     // [H]
+    float* state;           // slot s: state + s * slot_stride, [H][Dv][D]
+    const int* entry_start;
+    const int* slots;
+    float* o;               // [n][H][Dv]
+    long long slot_stride, ldb;
+    int H, G, D, Dv;
+};
+
+// vt_general_delta's arrangement: 16 rows of lanes for the recurrence (a row per value column, lane r holding the DS
+// consecutive state elements from d = DS r) and TILE tokens x 16 lanes for a tile's inputs.  Per token and column, with
+// k' and q' the unit vectors (q' also times D^-1/2):
+//     S_d <- g_d S_d;  p = k' . S;  u = beta (v - p);  S_d <- S_d + k'_d u;  o = q' . S
+// the same instructions in the same order whatever the tile, so nothing depends on how a request was cut.
+template <typename TI, typename TB, int DS, int TILE>
+__global__ __launch_bounds__(256) void delta_rule_channel_kernel(ChannelDeltaArgs a) {
+    constexpr int DP = 16 * DS;
+    __shared__ __attribute__((aligned(16))) float qs[TILE][DP];      // unit queries times D^-1/2
+    __shared__ __attribute__((aligned(16))) float ks[TILE][DP];      // unit keys
+    __shared__ __attribute__((aligned(16))) float gs[TILE][DP];      // decays
+    __shared__ float vs[TILE][DELTA_GROUPS];
+    __shared__ float beta_s[TILE];
+
+    const int e = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * DELTA_GROUPS;
+    const int tid = threadIdx.x;
+    const int r = tid & 15, cl = tid >> 4;
+    const int D = a.D, Dv = a.Dv, H = a.H, G = a.G;
+    const int kh = h / (H / G);
+    const int C = 2 * G * D + H * Dv;
+    const int start = a.entry_start[e], end = a.entry_start[e + 1];
+    float* S_head = a.state + (size_t)a.slots[e] * a.slot_stride + (size_t)h * Dv * D;
+    const TI* x = (const TI*)a.qkv;
+    const TB* bl = (const TB*)a.beta;
+    const int col = col0 + cl;
+    const float decay_rate = expf(a.a_log[h]);
+    const float q_scale = 1.0f / sqrtf((float)D);
+
+    float S[DS];
+#pragma unroll
+    for (int i = 0; i < DS; ++i) {
+        const int d = DS * r + i;
+        S[i] = (col < Dv && d < D) ? S_head[(size_t)col * D + d] : 0.f;
+    }
+
+    float in_q[DS], in_k[DS], in_z[DS], in_v = 0.f, in_b = 0.f;
+    auto fetch = [&](int t0) {
+        const int t = t0 + cl;
+        const bool ok = cl < TILE && t < end;
+        const size_t row = (size_t)(ok ? t : start) * C;
+        const size_t zrow = (size_t)(ok ? t : start) * H * D + (size_t)h * D;
+#pragma unroll
+        for (int i = 0; i < DS; ++i) {
+            const int d = DS * r + i;
+            const bool in = ok && d < D;
+            in_q[i] = in ? load_f32<TI>(x, row + (size_t)kh * D + d) : 0.f;
+            in_k[i] = in ? load_f32<TI>(x, row + (size_t)(G + kh) * D + d) : 0.f;
+            in_z[i] = in ? a.z[zrow + d] : 0.f;
+        }
+        const int j = col0 + r;
+        in_v = (ok && j < Dv) ? load_f32<TI>(x, row + (size_t)2 * G * D + (size_t)h * Dv + j) : 0.f;
+        in_b = (ok && r == 0) ? load_f32<TB>(bl, (size_t)t * a.ldb + h) : 0.f;
+    };
+    fetch(start);
+    for (int t0 = start; t0 < end; t0 += TILE) {
+        const int nt = min(TILE, end - t0);
+        __syncthreads();        // the tile before has been read
+        if (cl < TILE) {
+            float sq = 0.f, sk = 0.f;
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                sq = fmaf(in_q[i], in_q[i], sq);
+                sk = fmaf(in_k[i], in_k[i], sk);
+            }
+            sq = row16_sum(sq);
+            sk = row16_sum(sk);
+            const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                const int d = DS * r + i;
+                qs[cl][d] = in_q[i] * rq;
+                ks[cl][d] = in_k[i] * rk;
+                gs[cl][d] = expf(-decay_rate * softplus_f(in_z[i]));
+            }
+            vs[cl][r] = in_v;
+            if (r == 0) beta_s[cl] = 1.0f / (1.0f + expf(-in_b));
+        }
+        __syncthreads();
+        if (t0 + TILE < end) fetch(t0 + TILE);      // on its way while this tile is worked through
+        auto token = [&](int tt) {
+            float p = 0.f;
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                const int d = DS * r + i;
+                S[i] *= gs[tt][d];
+                p = fmaf(ks[tt][d], S[i], p);
+            }
+            p = row16_sum(p);
+            const float u = beta_s[tt] * (vs[tt][cl] - p);
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                const int d = DS * r + i;
+                S[i] = fmaf(ks[tt][d], u, S[i]);
+                acc = fmaf(qs[tt][d], S[i], acc);
+            }
+            acc = row16_sum(acc);
+            if (r == 0 && col < Dv) a.o[((size_t)(t0 + tt) * H + h) * Dv + col] = acc;
+        };
+        if (nt == TILE) {
+#pragma unroll
+            for (int tt = 0; tt < TILE; ++tt) token(tt);
+        } else {
+            for (int tt = 0; tt < nt; ++tt) token(tt);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < DS; ++i) {
+        const int d = DS * r + i;
+        if (col < Dv && d < D) S_head[(size_t)col * D + d] = S[i];
+    }
+}
+
+extern "C" int vt_delta_rule_channel(const void* qkv, int dtype, const void* beta, int beta_dtype, long long ldb,
+                                     const float* z, const float* a_log, float* state, long long slot_stride,
+                                     const int* entry_start, const int* slots, float* o, int n_entries, int H, int G, int D,
+                                     int Dv, hipStream_t stream) {
+    VT_REQUIRE(n_entries >= 0 && H > 0 && G > 0 && H % G == 0, "vt_delta_rule_channel: bad heads %d/%d", H, G);
+    VT_REQUIRE(D > 0 && D <= 256 && Dv > 0, "vt_delta_rule_channel: head sizes %d/%d (keys up to 256)", D, Dv);
+    VT_REQUIRE(slot_stride >= (long long)H * D * Dv, "vt_delta_rule_channel: state slots are too short");
+    VT_REQUIRE(ldb >= H, "vt_delta_rule_channel: rows of write-strength logits are too short");
+    VT_REQUIRE(H <= 65535, "vt_delta_rule_channel: too many heads (%d)", H);
+    if (n_entries == 0) return 0;
+    ChannelDeltaArgs a;
+    a.qkv = qkv; a.beta = beta; a.z = z; a.a_log = a_log; a.state = state; a.entry_start = entry_start; a.slots = slots;
+    a.o = o; a.slot_stride = slot_stride; a.ldb = ldb; a.H = H; a.G = G; a.D = D; a.Dv = Dv;
+    const int share = (D + 15) / 16;
+    const dim3 grid(n_entries, H, (Dv + DELTA_GROUPS - 1) / DELTA_GROUPS);
+#define VT_CDELTA(TI, TB)                                                                                  \
+    do {                                                                                                   \
+        if (share <= 1) delta_rule_channel_kernel<TI, TB, 1, 16><<<grid, 256, 0, stream>>>(a);             \
+        else if (share <= 2) delta_rule_channel_kernel<TI, TB, 2, 16><<<grid, 256, 0, stream>>>(a);        \
+        else if (share <= 4) delta_rule_channel_kernel<TI, TB, 4, 16><<<grid, 256, 0, stream>>>(a);        \
+        else if (share <= 8) delta_rule_channel_kernel<TI, TB, 8, 16><<<grid, 256, 0, stream>>>(a);        \
+        else delta_rule_channel_kernel<TI, TB, 16, 16><<<grid, 256, 0, stream>>>(a);                       \
+    } while (0)
+    if (dtype == VT_F32 && beta_dtype == VT_F32) VT_CDELTA(float, float);
+    else if (dtype == VT_BF16 && beta_dtype == VT_F32) VT_CDELTA(bf16_t, float);
+    else if (dtype == VT_BF16 && beta_dtype == VT_BF16) VT_CDELTA(bf16_t, bf16_t);
+    else return vt_fail("vt_delta_rule_channel: dtypes %d / %d are not handled", dtype, beta_dtype);
+#undef VT_CDELTA
+    VT_CHECK_LAUNCH("vt_delta_rule_channel");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+struct MemoryArgs {
+    const void* x;          // [n][ldx]: per head D queries from q_col, D keys from k_col, Dv values from v_col, and one
+                            // logit per head of the input gate from i_col and of the forget gate from f_col
+    const float* i_bias;    // [H] or null
+    const float* f_bias;    // [H] or null
+    float* state;           // slot s: state + s * slot_stride: [H][Dv][D] matrices, then [H][ZB][D] normalizers, then
+                            // [H][ZB] maxima, ZB = blocks of 16 value columns
+    const int* entry_start;
+    const int* slots;
+    float* o;               // [n][H][Dv]
+    long long ldx, slot_stride;
+    int q_col, k_col, v_col, i_col, f_col;
+    int H, D, Dv;
+    float cap, q_scale;
+};
+
+__device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+template <typename TI, int DS, int TILE>
+__global__ __launch_bounds__(256) void matrix_memory_kernel(MemoryArgs a) {
+    constexpr int DP = 16 * DS;
+    __shared__ __attribute__((aligned(16))) float qs[TILE][DP];
+    __shared__ __attribute__((aligned(16))) float ks[TILE][DP];
+    __shared__ float vs[TILE][DELTA_GROUPS];
+    __shared__ float i_s[TILE], f_s[TILE];
+
+    const int e = blockIdx.x, h = blockIdx.y, zb = blockIdx.z, col0 = zb * DELTA_GROUPS;
+    const int ZB = gridDim.z;
+    const int tid = threadIdx.x;
+    const int r = tid & 15, cl = tid >> 4;
+    const int D = a.D, Dv = a.Dv, H = a.H;
+    const int start = a.entry_start[e], end = a.entry_start[e + 1];
+    float* slot = a.state + (size_t)a.slots[e] * a.slot_stride;
+    float* S_head = slot + (size_t)h * Dv * D;
+    float* n_own = slot + (size_t)H * Dv * D + ((size_t)h * ZB + zb) * D;
+    float* m_own = slot + (size_t)H * Dv * D + (size_t)H * ZB * D + (size_t)h * ZB + zb;
+    const TI* x = (const TI*)a.x;
+    const int col = col0 + cl;
+    const float ib = a.i_bias ? a.i_bias[h] : 0.f, fb = a.f_bias ? a.f_bias[h] : 0.f;
+
+    float S[DS], nn[DS];
+#pragma unroll
+    for (int i = 0; i < DS; ++i) {
+        const int d = DS * r + i;
+        S[i] = (col < Dv && d < D) ? S_head[(size_t)col * D + d] : 0.f;
+        nn[i] = d < D ? n_own[d] : 0.f;
+    }
+    float m = *m_own;
+
+    float in_q[DS], in_k[DS], in_v = 0.f, in_i = 0.f, in_f = 0.f;
+    auto fetch = [&](int t0) {
+        const int t = t0 + cl;
+        const bool ok = cl < TILE && t < end;
+        const size_t row = (size_t)(ok ? t : start) * a.ldx;
+#pragma unroll
+        for (int i = 0; i < DS; ++i) {
+            const int d = DS * r + i;
+            const bool in = ok && d < D;
+            in_q[i] = in ? load_f32<TI>(x, row + a.q_col + (size_t)h * D + d) : 0.f;
+            in_k[i] = in ? load_f32<TI>(x, row + a.k_col + (size_t)h * D + d) : 0.f;
+        }
+        const int j = col0 + r;
+        in_v = (ok && j < Dv) ? load_f32<TI>(x, row + a.v_col + (size_t)h * Dv + j) : 0.f;
+        if (ok && r == 0) {
+            in_i = load_f32<TI>(x, row + a.i_col + h);
+            in_f = load_f32<TI>(x, row + a.f_col + h);
+        }
+    };
+    fetch(start);
+    for (int t0 = start; t0 < end; t0 += TILE) {
+        const int nt = min(TILE, end - t0);
+        __syncthreads();        // the tile before has been read
+        if (cl < TILE) {
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                const int d = DS * r + i;
+                qs[cl][d] = in_q[i] * a.q_scale;
+                ks[cl][d] = in_k[i];
+            }
+            vs[cl][r] = in_v;
+            if (r == 0) {
+                // the gates' logarithms, capped (cap 0: as they come)
+                const float zi = in_i + ib, zf = in_f + fb;
+                i_s[cl] = a.cap > 0.f ? a.cap * tanhf(zi / a.cap) : zi;
+                f_s[cl] = log_sigmoid_f(a.cap > 0.f ? a.cap * tanhf(zf / a.cap) : zf);
+            }
+        }
+        __syncthreads();
+        if (t0 + TILE < end) fetch(t0 + TILE);      // on its way while this tile is worked through
+        auto token = [&](int tt) {
+            const float lf = f_s[tt] + m, li = i_s[tt];
+            const float m_new = fmaxf(lf, li);
+            const float keep = expf(lf - m_new), put = expf(li - m_new);
+            m = m_new;
+            const float pv = put * vs[tt][cl];
+            float acc = 0.f, den = 0.f;
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                const int d = DS * r + i;
+                const float kd = ks[tt][d], qd = qs[tt][d];
+                S[i] = fmaf(keep, S[i], kd * pv);
+                nn[i] = fmaf(keep, nn[i], kd * put);
+                acc = fmaf(qd, S[i], acc);
+                den = fmaf(qd, nn[i], den);
+            }
+            acc = row16_sum(acc);
+            den = row16_sum(den);
+            if (r == 0 && col < Dv)
+                a.o[((size_t)(t0 + tt) * H + h) * Dv + col] = acc / (fmaxf(fabsf(den), expf(-m_new)) + 1e-6f);
+        };
+        if (nt == TILE) {
+#pragma unroll
+            for (int tt = 0; tt < TILE; ++tt) token(tt);
+        } else {
+            for (int tt = 0; tt < nt; ++tt) token(tt);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < DS; ++i) {
+        const int d = DS * r + i;
+        if (col < Dv && d < D) S_head[(size_t)col * D + d] = S[i];
+        if (cl == 0 && d < D) n_own[d] = nn[i];
+    }
+    if (tid == 0) *m_own = m;
+}
+
+extern "C" long long vt_matrix_memory_state_floats(int H, int D, int Dv) {
+    const long long zb = (Dv + DELTA_GROUPS - 1) / DELTA_GROUPS;
+    return (long long)H * Dv * D + (long long)H * zb * D + (long long)H * zb;
+}
+
+extern "C" int vt_matrix_memory(const void* x, int dtype, long long ldx, int q_col, int k_col, int v_col, int i_col, int f_col,
+                                const float* i_bias, const float* f_bias, float* state, long long slot_stride,
+                                const int* entry_start, const int* slots, float* o, int n_entries, int H, int D, int Dv,
+                                float cap, float q_scale, hipStream_t stream) {
+    VT_REQUIRE(n_entries >= 0 && H > 0 && H <= 65535, "vt_matrix_memory: bad heads %d", H);
+    VT_REQUIRE(D > 0 && D <= 256 && Dv > 0, "vt_matrix_memory: head sizes %d/%d (keys up to 256)", D, Dv);
+    VT_REQUIRE(slot_stride >= vt_matrix_memory_state_floats(H, D, Dv), "vt_matrix_memory: state slots are too short");
+    VT_REQUIRE(min(min(q_col, k_col), min(v_col, min(i_col, f_col))) >= 0 && ldx >= max(q_col, k_col) + (long long)H * D &&
+               ldx >= v_col + (long long)H * Dv && ldx >= max(i_col, f_col) + (long long)H,
+               "vt_matrix_memory: rows are too short for their columns");
+    VT_REQUIRE(cap >= 0.f, "vt_matrix_memory: a negative cap");
+    if (n_entries == 0) return 0;
+    MemoryArgs a;
+    a.x = x; a.i_bias = i_bias; a.f_bias = f_bias; a.state = state; a.entry_start = entry_start; a.slots = slots; a.o = o;
+    a.ldx = ldx; a.slot_stride = slot_stride; a.q_col = q_col; a.k_col = k_col; a.v_col = v_col; a.i_col = i_col; a.f_col = f_col;
+    a.H = H; a.D = D; a.Dv = Dv; a.cap = cap; a.q_scale = q_scale;
+    const int share = (D + 15) / 16;
+    const dim3 grid(n_entries, H, (Dv + DELTA_GROUPS - 1) / DELTA_GROUPS);
+#define VT_MEMORY(TI)                                                                              \
+    do {                                                                                           \
+        if (share <= 1) matrix_memory_kernel<TI, 1, 16><<<grid, 256, 0, stream>>>(a);              \
+        else if (share <= 2) matrix_memory_kernel<TI, 2, 16><<<grid, 256, 0, stream>>>(a);         \
+        else if (share <= 4) matrix_memory_kernel<TI, 4, 16><<<grid, 256, 0, stream>>>(a);         \
+        else if (share <= 8) matrix_memory_kernel<TI, 8, 16><<<grid, 256, 0, stream>>>(a);         \
+        else matrix_memory_kernel<TI, 16, 16><<<grid, 256, 0, stream>>>(a);                        \
+    } while (0)
+    if (dtype == VT_F32) VT_MEMORY(float);
+    else if (dtype == VT_BF16) VT_MEMORY(bf16_t);
+    else return vt_fail("vt_matrix_memory: unknown dtype %d", dtype);
+#undef VT_MEMORY
+    VT_CHECK_LAUNCH("vt_matrix_memory");
     return 0;
 }

@@ -182,6 +182,195 @@ extern "C" int vt_rmsnorm(float* h, const void* delta, int delta_dtype, const fl
 }
 
 // ---------------------------------------------------------------------------
+// Layer norm with gain and bias, fused with the residual additions in front of it:
+//     x = h[row] + (delta[row] + delta2[row]);   out = (x - mean) / sqrt(var + eps) * gain + bias
+// with var the mean of the squared deviations from the mean (two sums, the second over x - mean), all in float32.
+// A thread keeps its values in registers between the sums and the scaling (up to LN_MAXV * 256 columns; wider rows
+// are read again).  With `update` the sum x is written back to h.
+// ---------------------------------------------------------------------------
+#define LN_MAXV 16
+template <typename TD, typename TO, int NV>
+__global__ __launch_bounds__(256) void layernorm_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                       const TD* __restrict__ delta2, const float* __restrict__ gain,
+                                                       const float* __restrict__ bias, TO* __restrict__ out,
+                                                       const int* __restrict__ rows, int hidden, float eps, int update) {
+    __shared__ float red[16];
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    float* hr = h + src * hidden;
+    const TD* d1 = delta ? delta + src * hidden : nullptr;
+    const TD* d2 = delta2 ? delta2 + src * hidden : nullptr;
+    auto value = [&](int i) -> float {
+        float x = hr[i];
+        if (d1 && d2) x += load_f32<TD>(d1, i) + load_f32<TD>(d2, i);
+        else if (d1) x += load_f32<TD>(d1, i);
+        return x;
+    };
+    float x[NV > 0 ? NV : 1];
+    float sum = 0.f;
+    if (NV > 0) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int i = tid + v * 256;
+            x[v] = i < hidden ? value(i) : 0.f;
+            if (i < hidden && update && d1) hr[i] = x[v];
+            sum += x[v];
+        }
+    } else {
+        for (int i = tid; i < hidden; i += 256) {
+            const float xv = value(i);
+            if (update && d1) hr[i] = xv;
+            sum += xv;
+        }
+        __syncthreads();
+        d1 = update && d1 ? nullptr : d1;       // (h now holds the sum)
+        if (!d1) d2 = nullptr;
+    }
+    const float mean = block_sum(sum, red) / (float)hidden;
+    float sq = 0.f;
+    if (NV > 0) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int i = tid + v * 256;
+            const float dv = i < hidden ? x[v] - mean : 0.f;
+            sq = fmaf(dv, dv, sq);
+        }
+    } else {
+        for (int i = tid; i < hidden; i += 256) {
+            const float dv = value(i) - mean;
+            sq = fmaf(dv, dv, sq);
+        }
+    }
+    const float rinv = 1.0f / sqrtf(block_sum(sq, red) / (float)hidden + eps);
+    TO* o = out + (size_t)r * hidden;
+    if (NV > 0) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int i = tid + v * 256;
+            if (i < hidden) store_f32<TO>(o, i, fmaf((x[v] - mean) * rinv, gain[i], bias ? bias[i] : 0.f));
+        }
+    } else {
+        for (int i = tid; i < hidden; i += 256)
+            store_f32<TO>(o, i, fmaf((value(i) - mean) * rinv, gain[i], bias ? bias[i] : 0.f));
+    }
+}
+
+template <typename TD, typename TO>
+static void launch_layernorm(float* h, const void* delta, const void* delta2, const float* gain, const float* bias, void* out,
+                             const int* rows, int n_out, int hidden, float eps, int update_h, hipStream_t stream) {
+#define VT_LN(NV) layernorm_kernel<TD, TO, NV><<<n_out, 256, 0, stream>>>(h, (const TD*)delta, (const TD*)delta2, gain, bias, \
+                                                                         (TO*)out, rows, hidden, eps, update_h)
+    if (hidden <= 256) VT_LN(1);
+    else if (hidden <= 512) VT_LN(2);
+    else if (hidden <= 1024) VT_LN(4);
+    else if (hidden <= 2048) VT_LN(8);
+    else if (hidden <= 256 * LN_MAXV) VT_LN(LN_MAXV);
+    else VT_LN(0);
+#undef VT_LN
+}
+
+extern "C" int vt_layernorm(float* h, const void* delta, const void* delta2, int delta_dtype, const float* gain,
+                            const float* bias, void* out, int out_dtype, const int* rows, int n_out, int hidden, float eps,
+                            int update_h, hipStream_t stream) {
+    VT_REQUIRE(n_out >= 0 && hidden > 0, "vt_layernorm: bad sizes n=%d hidden=%d", n_out, hidden);
+    VT_REQUIRE(!(update_h && rows), "vt_layernorm: cannot update the residual through a row list");
+    VT_REQUIRE(delta || !delta2, "vt_layernorm: a second addend without a first");
+    if (n_out == 0) return 0;
+#define VT_LNL(TD, TO) launch_layernorm<TD, TO>(h, delta, delta2, gain, bias, out, rows, n_out, hidden, eps, update_h, stream)
+    const int dd = delta ? delta_dtype : VT_F32;
+    if (dd == VT_F32 && out_dtype == VT_F32) VT_LNL(float, float);
+    else if (dd == VT_F32 && out_dtype == VT_BF16) VT_LNL(float, bf16_t);
+    else if (dd == VT_BF16 && out_dtype == VT_BF16) VT_LNL(bf16_t, bf16_t);
+    else if (dd == VT_BF16 && out_dtype == VT_F32) VT_LNL(bf16_t, float);
+    else return vt_fail("vt_layernorm: dtypes %d -> %d are not handled", delta_dtype, out_dtype);
+#undef VT_LNL
+    VT_CHECK_LAUNCH("vt_layernorm");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Small passes over whole rows for layers whose sublayers run side by side and for a stream that is re-entered:
+//   vt_residual_add2: h += (a + b)                               two results joined first, then added to the stream
+//   vt_scaled_sum:    out = sa * a + sb * b  (float32 out)       two mixers side by side, each with a constant factor
+//   vt_concat_cast:   out[t] = [a[t] | b[t]] in out's type       two float32 streams as one product's input
+//   vt_set_plus_row:  h[t] = y[t] + row (row may be null)        the stream replaced by a product's result plus a vector
+// ---------------------------------------------------------------------------
+template <typename TD>
+__global__ void residual_add2_kernel(float* __restrict__ h, const TD* __restrict__ a, const TD* __restrict__ b, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) h[i] += load_f32<TD>(a, i) + load_f32<TD>(b, i);
+}
+extern "C" int vt_residual_add2(float* h, const void* a, const void* b, int dtype, long long n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == VT_F32) residual_add2_kernel<float><<<blocks, 256, 0, stream>>>(h, (const float*)a, (const float*)b, (size_t)n);
+    else if (dtype == VT_BF16) residual_add2_kernel<bf16_t><<<blocks, 256, 0, stream>>>(h, (const bf16_t*)a, (const bf16_t*)b, (size_t)n);
+    else return vt_fail("vt_residual_add2: unknown dtype %d", dtype);
+    VT_CHECK_LAUNCH("vt_residual_add2");
+    return 0;
+}
+
+template <typename TA, typename TB>
+__global__ void scaled_sum_kernel(const TA* __restrict__ a, float sa, const TB* __restrict__ b, float sb,
+                                  float* __restrict__ out, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = fmaf(sb, load_f32<TB>(b, i), sa * load_f32<TA>(a, i));
+}
+extern "C" int vt_scaled_sum(const void* a, int a_dtype, float sa, const void* b, int b_dtype, float sb, float* out,
+                             long long n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (a_dtype == VT_F32 && b_dtype == VT_F32) scaled_sum_kernel<float, float><<<blocks, 256, 0, stream>>>((const float*)a, sa, (const float*)b, sb, out, (size_t)n);
+    else if (a_dtype == VT_BF16 && b_dtype == VT_BF16) scaled_sum_kernel<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)a, sa, (const bf16_t*)b, sb, out, (size_t)n);
+    else if (a_dtype == VT_F32 && b_dtype == VT_BF16) scaled_sum_kernel<float, bf16_t><<<blocks, 256, 0, stream>>>((const float*)a, sa, (const bf16_t*)b, sb, out, (size_t)n);
+    else if (a_dtype == VT_BF16 && b_dtype == VT_F32) scaled_sum_kernel<bf16_t, float><<<blocks, 256, 0, stream>>>((const bf16_t*)a, sa, (const float*)b, sb, out, (size_t)n);
+    else return vt_fail("vt_scaled_sum: dtypes %d / %d are not handled", a_dtype, b_dtype);
+    VT_CHECK_LAUNCH("vt_scaled_sum");
+    return 0;
+}
+
+template <typename TO>
+__global__ void concat_cast_kernel(const float* __restrict__ a, const float* __restrict__ b, TO* __restrict__ out,
+                                   size_t n, int wa, int wb) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t t = i / (size_t)(wa + wb);
+    const int c = (int)(i - t * (size_t)(wa + wb));
+    store_f32<TO>(out, i, c < wa ? a[t * wa + c] : b[t * wb + (c - wa)]);
+}
+extern "C" int vt_concat_cast(const float* a, const float* b, void* out, int out_dtype, long long tokens, int wa, int wb,
+                              hipStream_t stream) {
+    VT_REQUIRE(tokens >= 0 && wa > 0 && wb > 0, "vt_concat_cast: bad sizes %lld x (%d + %d)", tokens, wa, wb);
+    const long long n = tokens * (wa + wb);
+    if (n <= 0) return 0;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (out_dtype == VT_F32) concat_cast_kernel<float><<<blocks, 256, 0, stream>>>(a, b, (float*)out, (size_t)n, wa, wb);
+    else if (out_dtype == VT_BF16) concat_cast_kernel<bf16_t><<<blocks, 256, 0, stream>>>(a, b, (bf16_t*)out, (size_t)n, wa, wb);
+    else return vt_fail("vt_concat_cast: unknown dtype %d", out_dtype);
+    VT_CHECK_LAUNCH("vt_concat_cast");
+    return 0;
+}
+
+template <typename TY>
+__global__ void set_plus_row_kernel(float* __restrict__ h, const TY* __restrict__ y, const float* __restrict__ row,
+                                    size_t n, int hidden) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) h[i] = load_f32<TY>(y, i) + (row ? row[i % (size_t)hidden] : 0.f);
+}
+extern "C" int vt_set_plus_row(float* h, const void* y, int y_dtype, const float* row, long long tokens, int hidden,
+                               hipStream_t stream) {
+    VT_REQUIRE(hidden > 0 && tokens >= 0, "vt_set_plus_row: bad sizes %lld x %d", tokens, hidden);
+    const long long n = tokens * hidden;
+    if (n <= 0) return 0;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (y_dtype == VT_F32) set_plus_row_kernel<float><<<blocks, 256, 0, stream>>>(h, (const float*)y, row, (size_t)n, hidden);
+    else if (y_dtype == VT_BF16) set_plus_row_kernel<bf16_t><<<blocks, 256, 0, stream>>>(h, (const bf16_t*)y, row, (size_t)n, hidden);
+    else return vt_fail("vt_set_plus_row: unknown dtype %d", y_dtype);
+    VT_CHECK_LAUNCH("vt_set_plus_row");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
 // h += delta (fp32 sum), for a residual that no norm follows
 // ---------------------------------------------------------------------------
 template <typename TD>
@@ -349,13 +538,15 @@ extern "C" int vt_silu_mul(const void* gu, int in_dtype, void* out, int out_dtyp
 // ---------------------------------------------------------------------------
 // A gated unit with bounds: g = min(gu[t, i], limit), u = clamp(gu[t, inter + i], -limit, limit),
 // out[t, i] = g * sigmoid(alpha * g * (1 + cubic * g^2)) * (u + shift).  limit <= 0: no bounds.  (alpha 1, shift 0,
-// cubic 0 and no bounds is vt_silu_mul; alpha 2 sqrt(2 / pi) and cubic 0.044715 is the tanh form of GELU.)  A thread takes four columns where the width is a multiple of 4.
+// cubic 0 and no bounds is vt_silu_mul; alpha 2 sqrt(2 / pi) and cubic 0.044715 is the tanh form of GELU; an infinite
+// alpha makes the sigmoid a step, which is ReLU: max(g, 0) * (u + shift).)  A thread takes four columns where the width is a multiple of 4.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float bounded_gate(float g, float u, float alpha, float limit, float shift, float cubic) {
     if (limit > 0.f) {
         g = fminf(g, limit);
         u = fminf(fmaxf(u, -limit), limit);
     }
+    if (isinf(alpha)) return fmaxf(g, 0.f) * (u + shift);       // the sigmoid as a step: ReLU
     const float z = cubic != 0.f ? alpha * g * fmaf(cubic * g, g, 1.f) : alpha * g;
     return g / (1.f + expf(-z)) * (u + shift);
 }
@@ -391,6 +582,7 @@ __device__ __forceinline__ float bounded_gate_fast(float g, float u, float alpha
         g = fminf(g, limit);
         u = fminf(fmaxf(u, -limit), limit);
     }
+    if (isinf(alpha)) return fmaxf(g, 0.f) * (u + shift);
     const float z = cubic != 0.f ? alpha * g * fmaf(cubic * g, g, 1.f) : alpha * g;
     return g * __builtin_amdgcn_rcpf(1.f + __expf(-z)) * (u + shift);
 }

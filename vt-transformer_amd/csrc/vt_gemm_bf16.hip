@@ -141,7 +141,8 @@ __device__ __forceinline__ bf16x8_t load_x(const bf16_t* row, int k, int K) {
 //     g <- min(g, limit), u <- clamp(u, -limit, limit)   (limit 0: no bounds);
 //     g * sigmoid(alpha * g * (1 + cubic * g^2)) * (u + shift).
 // alpha 1, limit 0, shift 0, cubic 0 is SiLU gating, to the bit what it was before the form had parameters;
-// alpha 2 sqrt(2 / pi), cubic 0.044715 is the tanh form of GELU, since (1 + tanh z) / 2 = sigmoid(2 z).
+// alpha 2 sqrt(2 / pi), cubic 0.044715 is the tanh form of GELU, since (1 + tanh z) / 2 = sigmoid(2 z);
+// an infinite alpha is ReLU.
 struct GateForm {
     float alpha, limit, shift, cubic;
 };
@@ -150,6 +151,7 @@ __device__ __forceinline__ float gate_form(float g, float u, const GateForm& f) 
         g = fminf(g, f.limit);
         u = fminf(fmaxf(u, -f.limit), f.limit);
     }
+    if (isinf(f.alpha)) return fmaxf(g, 0.f) * (u + f.shift);      // the sigmoid as a step: ReLU
     const float z = f.cubic != 0.f ? f.alpha * g * fmaf(f.cubic * g, g, 1.f) : f.alpha * g;
     return g / (1.f + expf(-z)) * (u + f.shift);
 }

@@ -147,6 +147,80 @@ def add_row(h: torch.Tensor, delta: Optional[torch.Tensor], row: torch.Tensor) -
     return h
 
 
+def layernorm(h: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tensor, bias: Optional[torch.Tensor],
+              out: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None, update_h: bool = True,
+              delta2: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[r] = (x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * gain + bias with x = h[row] + (delta[row] +
+    delta2[row]), everything in float32; with update_h the sum is written back to h."""
+    hidden = h.shape[-1]
+    _chk(h, "layernorm.h", torch.float32)
+    _chk(gain, "layernorm.gain", torch.float32, (hidden,))
+    if bias is not None:
+        _chk(bias, "layernorm.bias", torch.float32, (hidden,))
+    if delta is not None:
+        _chk(delta, "layernorm.delta", None, h.shape)
+    if delta2 is not None:
+        if delta is None:
+            raise KernelError("layernorm: a second addend without a first")
+        _chk(delta2, "layernorm.delta2", delta.dtype, h.shape)
+    if rows is not None:
+        _chk(rows, "layernorm.rows", torch.int32)
+        n_out = rows.numel()
+        update_h = False
+    else:
+        n_out = h.shape[0]
+    _chk(out, "layernorm.out", None, (n_out, hidden))
+    _run(load_lib("vt_elementwise", half=_half(delta, out)), "vt_layernorm", _ptr(h), _ptr(delta), _ptr(delta2),
+         _i(_code(delta) if delta is not None else F32), _ptr(gain), _ptr(bias), _ptr(out), _i(_code(out)), _ptr(rows),
+         _i(n_out), _i(hidden), _f(eps), _i(1 if (update_h and delta is not None) else 0), _stream())
+    return out
+
+
+def residual_add2(h: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """h += (a + b): two results joined first, then added to the float32 stream."""
+    _chk(h, "residual_add2.h", torch.float32)
+    _chk(a, "residual_add2.a", None, h.shape)
+    _chk(b, "residual_add2.b", a.dtype, h.shape)
+    _run(load_lib("vt_elementwise", half=_half(a)), "vt_residual_add2", _ptr(h), _ptr(a), _ptr(b), _i(_code(a)),
+         ctypes.c_longlong(h.numel()), _stream())
+    return h
+
+
+def scaled_sum(a: torch.Tensor, sa: float, b: torch.Tensor, sb: float, out: torch.Tensor) -> torch.Tensor:
+    """out = sa * a + sb * b, float32."""
+    _chk(a, "scaled_sum.a")
+    _chk(b, "scaled_sum.b", None, a.shape)
+    _chk(out, "scaled_sum.out", torch.float32, a.shape)
+    _run(load_lib("vt_elementwise", half=_half(a, b)), "vt_scaled_sum", _ptr(a), _i(_code(a)), _f(sa), _ptr(b), _i(_code(b)),
+         _f(sb), _ptr(out), ctypes.c_longlong(a.numel()), _stream())
+    return out
+
+
+def concat_cast(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = [a[t] | b[t]] in out's dtype, from two float32 tensors with the same rows."""
+    n = a.shape[0]
+    _chk(a, "concat_cast.a", torch.float32)
+    _chk(b, "concat_cast.b", torch.float32)
+    if a.dim() != 2 or b.dim() != 2 or b.shape[0] != n:
+        raise KernelError(f"concat_cast: shapes {tuple(a.shape)} and {tuple(b.shape)}")
+    _chk(out, "concat_cast.out", None, (n, a.shape[1] + b.shape[1]))
+    _run(load_lib("vt_elementwise", half=_half(out)), "vt_concat_cast", _ptr(a), _ptr(b), _ptr(out), _i(_code(out)),
+         ctypes.c_longlong(n), _i(a.shape[1]), _i(b.shape[1]), _stream())
+    return out
+
+
+def set_plus_row(h: torch.Tensor, y: torch.Tensor, row: Optional[torch.Tensor]) -> torch.Tensor:
+    """h[t] = y[t] + row (row None: h = y), for every token t: the float32 stream replaced."""
+    n, hidden = h.shape
+    _chk(h, "set_plus_row.h", torch.float32)
+    _chk(y, "set_plus_row.y", None, h.shape)
+    if row is not None:
+        _chk(row, "set_plus_row.row", torch.float32, (hidden,))
+    _run(load_lib("vt_elementwise", half=_half(y)), "vt_set_plus_row", _ptr(h), _ptr(y), _i(_code(y)), _ptr(row),
+         ctypes.c_longlong(n), _i(hidden), _stream())
+    return h
+
+
 def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     n, two_i = gu.shape
     _chk(gu, "silu_mul.gu")
@@ -729,16 +803,21 @@ def qk_prepare(x: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch
                k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], n_heads: int, n_kv: int, key_dim: int,
                value_dim: int, unit_rms_eps: Optional[float], write_kv: bool = True,
                q_temp: Optional[tuple] = None, v_first: Optional[torch.Tensor] = None,
-               v_lambda: Optional[torch.Tensor] = None) -> None:
+               v_lambda: Optional[torch.Tensor] = None, q_gain: Optional[torch.Tensor] = None,
+               k_gain: Optional[torch.Tensor] = None) -> None:
     """x [n, >= (H + G) D + G Dv]: query heads, key heads, value heads.  Rotates the leading 2 * cos.shape[1] elements
     of every query and key head by the tables' angles at `positions`, divides each head by its root mean square
     (eps inside the root) unless unit_rms_eps is None, writes queries to q_out [n, H * D] and, with write_kv, keys and
     values into their pages ([page][kv][slot][D] and, transposed, [page][kv][Dv][slot]).
     q_temp (coef, every): the queries of position p times 1 + coef ln(floor((p + 1) / every) + 1).
     v_first (float32 [n, G * Dv]): without v_lambda the tokens' values are left there as well; with v_lambda (one
-    float32 on the device) the pages get (1 - lambda) v + lambda v_first instead of v."""
+    float32 on the device) the pages get (1 - lambda) v + lambda v_first instead of v.
+    q_gain / k_gain (float32 [D], shared by the heads): a gain per element on the scaled queries / keys."""
     n = x.shape[0]
     _chk(x, "qk_prepare.x")
+    for g, name in ((q_gain, "q_gain"), (k_gain, "k_gain")):
+        if g is not None:
+            _chk(g, "qk_prepare." + name, torch.float32, (key_dim,))
     need = (n_heads + (n_kv if write_kv else 0)) * key_dim + (n_kv * value_dim if write_kv else 0)
     if x.dim() != 2 or x.shape[1] < need:
         raise KernelError(f"qk_prepare.x: shape {tuple(x.shape)}, need {need} columns")
@@ -785,19 +864,24 @@ def qk_prepare(x: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch
          _ptr(block_table), _i(max_blocks), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _i(_code(q_out)), _i(page_size),
          _i(num_pages), _i(n), _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _i(1 if write_kv else 0),
          _i(0 if unit_rms_eps is None else 1), _f(unit_rms_eps or 0.0), _f(coef), _i(every), _i(vmix), _ptr(v_first),
-         _ptr(v_lambda if vmix == 2 else None), _stream())
+         _ptr(v_lambda if vmix == 2 else None), _ptr(q_gain), _ptr(k_gain), _stream())
 
 
 def attention_masked(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, positions: torch.Tensor,
                      tok_entry: torch.Tensor, block_table: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int,
                      key_dim: int, value_dim: int, scale: float, cap: float = 0.0, window: int = 0, chunk: int = 0,
                      gate: Optional[torch.Tensor] = None, gate_column: int = 0, sink: Optional[torch.Tensor] = None,
-                     slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     slopes: Optional[torch.Tensor] = None, dist_log: Optional[tuple] = None,
+                     score_shift: Optional[torch.Tensor] = None, sigmoid_weights: bool = False,
+                     gate_wide: bool = False) -> torch.Tensor:
     """out [n, H * Dv] = softmax over the seen keys of cap * tanh(scale q.k / cap) (cap 0: scale q.k), times V, times
     sigmoid(gate[:, gate_column + head]) if `gate` (a 2-d tensor whose rows are the tokens') is given.  Key j is seen
     from position i if j <= i, i - j < window (0: unbounded) and j is in i's chunk of `chunk` positions (0: unbounded).
     slopes (float32 [H]): slopes[h] * (i - j) is taken off the score; sink (float32 [H]): exp(sink[h]) is added to the
-    softmax's denominator."""
+    softmax's denominator.  dist_log (r1, r2), float32 [H] each: r1[h] ln(1 + r2[h] (i - j)) is taken off the score;
+    score_shift (float32 [H]): a number per head added to every score; sigmoid_weights: the weight of a seen key is
+    sigmoid(score), nothing is normalized; gate_wide: the gate is one logit per output element, gate[:, gate_column +
+    head * Dv + d]."""
     n = q.shape[0]
     num_pages, kvh, page_size, d = k_pages.shape
     dt = q.dtype
@@ -813,19 +897,37 @@ def attention_masked(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
     gptr, gcode, ldg = ctypes.c_void_p(0), F32, 0
     if gate is not None:
         _chk(gate, "attention_masked.gate")
-        if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + n_heads:
-            raise KernelError(f"attention_masked.gate: shape {tuple(gate.shape)} has no {n_heads} columns from {gate_column}")
+        g_cols = n_heads * value_dim if gate_wide else n_heads
+        if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + g_cols:
+            raise KernelError(f"attention_masked.gate: shape {tuple(gate.shape)} has no {g_cols} columns from {gate_column}")
         if dt == torch.float32 and gate.dtype != torch.float32:
             raise KernelError("attention_masked: float32 attention takes float32 gates")
         gptr = ctypes.c_void_p(gate.data_ptr() + gate_column * gate.element_size())
         gcode, ldg = _code(gate), gate.stride(0)
     _per_head(sink, "attention_masked.sink", n_heads)
     _per_head(slopes, "attention_masked.slopes", n_heads)
+    r1, r2 = _score_forms("attention_masked", n_heads, dist_log, score_shift, sigmoid_weights, sink)
     _run(load_lib("vt_attn_masked", half=_half(q, gate)), "vt_attn_masked", _ptr(q), _ptr(k_pages), _ptr(v_pages), _i(_code(q)),
          _ptr(positions), _ptr(tok_entry), _ptr(block_table), gptr, _i(gcode), ctypes.c_longlong(ldg), _ptr(out), _i(n),
          _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _i(page_size), _i(block_table.shape[1]), _i(num_pages),
-         _i(window), _i(chunk), _f(scale), _f(cap), _ptr(sink), _ptr(slopes), _stream())
+         _i(window), _i(chunk), _f(scale), _f(cap), _ptr(sink), _ptr(slopes), _ptr(r1), _ptr(r2), _ptr(score_shift),
+         _i(1 if sigmoid_weights else 0), _i(1 if (gate_wide and gate is not None) else 0), _stream())
     return out
+
+
+def _score_forms(who: str, n_heads: int, dist_log, score_shift, sigmoid_weights: bool, sink):
+    """Checks of the score's optional forms that the three masked attention kernels share; returns (r1, r2)."""
+    r1 = r2 = None
+    if dist_log is not None:
+        r1, r2 = dist_log
+        _per_head(r1, who + ".dist_log[0]", n_heads)
+        _per_head(r2, who + ".dist_log[1]", n_heads)
+        if r1 is None or r2 is None:
+            raise KernelError(who + ": the distance bias takes both of its numbers per head")
+    _per_head(score_shift, who + ".score_shift", n_heads)
+    if sigmoid_weights and sink is not None:
+        raise KernelError(who + ": sigmoid weights have no denominator for a sink to join")
+    return r1, r2
 
 
 def _per_head(t: Optional[torch.Tensor], name: str, n_heads: int) -> None:
@@ -844,7 +946,9 @@ def attention_masked_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch
                           n_heads: int, n_kv: int, key_dim: int, value_dim: int, scale: float, cap: float = 0.0,
                           window: int = 0, chunk: int = 0, gate: Optional[torch.Tensor] = None,
                           gate_column: int = 0, sink: Optional[torch.Tensor] = None,
-                          slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                          slopes: Optional[torch.Tensor] = None, dist_log: Optional[tuple] = None,
+                          score_shift: Optional[torch.Tensor] = None, sigmoid_weights: bool = False,
+                          gate_wide: bool = False) -> torch.Tensor:
     """attention_masked for the 16-bit types on the matrix cores.  tiles: int32 [n_tiles, 2], (first row, rows) of
     runs of up to 16 consecutive tokens of one request that together cover every token of the step once."""
     n = q.shape[0]
@@ -866,17 +970,20 @@ def attention_masked_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch
     gptr, gcode, ldg = ctypes.c_void_p(0), F32, 0
     if gate is not None:
         _chk(gate, "attention_masked_mfma.gate")
-        if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + n_heads:
-            raise KernelError(f"attention_masked_mfma.gate: shape {tuple(gate.shape)} has no {n_heads} columns from {gate_column}")
+        g_cols = n_heads * value_dim if gate_wide else n_heads
+        if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + g_cols:
+            raise KernelError(f"attention_masked_mfma.gate: shape {tuple(gate.shape)} has no {g_cols} columns from {gate_column}")
         gptr = ctypes.c_void_p(gate.data_ptr() + gate_column * gate.element_size())
         gcode, ldg = _code(gate), gate.stride(0)
     _per_head(sink, "attention_masked_mfma.sink", n_heads)
     _per_head(slopes, "attention_masked_mfma.slopes", n_heads)
+    r1, r2 = _score_forms("attention_masked_mfma", n_heads, dist_log, score_shift, sigmoid_weights, sink)
     _run(load_lib("vt_attn_masked_mfma", (key_dim, value_dim), half=_half(q, gate)), "vt_attn_masked_mfma", _ptr(q), _ptr(k_pages),
          _ptr(v_pages), _ptr(positions), _ptr(tok_entry), _ptr(block_table), _ptr(tiles), _i(tiles.numel() // 2), gptr,
          _i(gcode), ctypes.c_longlong(ldg), _ptr(out), _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _i(page_size),
          _i(block_table.shape[1]), _i(num_pages), _i(window), _i(chunk), _f(scale), _f(cap), _ptr(sink), _ptr(slopes),
-         _stream())
+         _ptr(r1), _ptr(r2), _ptr(score_shift), _i(1 if sigmoid_weights else 0),
+         _i(1 if (gate_wide and gate is not None) else 0), _stream())
     return out
 
 
@@ -893,7 +1000,9 @@ def attention_masked_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
                             splits: int, n_heads: int, n_kv: int, key_dim: int, value_dim: int, scale: float,
                             cap: float = 0.0, window: int = 0, chunk: int = 0, gate: Optional[torch.Tensor] = None,
                             gate_column: int = 0, sink: Optional[torch.Tensor] = None,
-                            slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                            slopes: Optional[torch.Tensor] = None, dist_log: Optional[tuple] = None,
+                            score_shift: Optional[torch.Tensor] = None, sigmoid_weights: bool = False,
+                            gate_wide: bool = False) -> torch.Tensor:
     """attention_masked for steps of single tokens in the 16-bit types on the matrix cores: the rows of a product are
     the query heads that share a key/value head.  part: float32 scratch of attention_masked_decode_scratch floats."""
     n = q.shape[0]
@@ -913,17 +1022,20 @@ def attention_masked_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     gptr, gcode, ldg = ctypes.c_void_p(0), F32, 0
     if gate is not None:
         _chk(gate, "attention_masked_decode.gate")
-        if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + n_heads:
-            raise KernelError(f"attention_masked_decode.gate: shape {tuple(gate.shape)} has no {n_heads} columns from {gate_column}")
+        g_cols = n_heads * value_dim if gate_wide else n_heads
+        if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + g_cols:
+            raise KernelError(f"attention_masked_decode.gate: shape {tuple(gate.shape)} has no {g_cols} columns from {gate_column}")
         gptr = ctypes.c_void_p(gate.data_ptr() + gate_column * gate.element_size())
         gcode, ldg = _code(gate), gate.stride(0)
     _per_head(sink, "attention_masked_decode.sink", n_heads)
     _per_head(slopes, "attention_masked_decode.slopes", n_heads)
+    r1, r2 = _score_forms("attention_masked_decode", n_heads, dist_log, score_shift, sigmoid_weights, sink)
     _run(load_lib("vt_attn_masked_mfma", (key_dim, value_dim), half=_half(q, gate)), "vt_attn_masked_decode", _ptr(q),
          _ptr(k_pages), _ptr(v_pages), _ptr(positions), _ptr(tok_entry), _ptr(block_table), gptr, _i(gcode),
          ctypes.c_longlong(ldg), _ptr(out), _ptr(part), ctypes.c_longlong(part.numel()), _i(splits), _i(n), _i(n_heads),
          _i(n_kv), _i(key_dim), _i(value_dim), _i(page_size), _i(block_table.shape[1]), _i(num_pages), _i(window), _i(chunk),
-         _f(scale), _f(cap), _ptr(sink), _ptr(slopes), _stream())
+         _f(scale), _f(cap), _ptr(sink), _ptr(slopes), _ptr(r1), _ptr(r2), _ptr(score_shift), _i(1 if sigmoid_weights else 0),
+         _i(1 if (gate_wide and gate is not None) else 0), _stream())
     return out
 
 
@@ -1126,9 +1238,11 @@ def gated_rmsnorm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, gat
     return out
 
 
-def lowrank_tanh(x: torch.Tensor, x_column: int, w2: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+def lowrank_tanh(x: torch.Tensor, x_column: int, w2: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                 tanh: bool = True) -> torch.Tensor:
     """out[t, j] = bias[j] + sum_l w2[j, l] * tanh(x[t, x_column + l]): float32 sums in the order of l, float32 results.
-    x: a 2-d tensor whose rows are the tokens'; w2 [M, L] in float32 or the 16-bit type."""
+    x: a 2-d tensor whose rows are the tokens'; w2 [M, L] in float32 or the 16-bit type.  tanh False: the low-rank part
+    enters as it is (the second half of a linear low-rank projection, kept in float32)."""
     n = x.shape[0]
     m, low = w2.shape
     _chk(x, "lowrank_tanh.x")
@@ -1142,7 +1256,7 @@ def lowrank_tanh(x: torch.Tensor, x_column: int, w2: torch.Tensor, bias: Optiona
     _chk(out, "lowrank_tanh.out", torch.float32, (n, m))
     xptr = ctypes.c_void_p(x.data_ptr() + x_column * x.element_size())
     _run(load_lib("vt_delta", half=_half(x, w2)), "vt_lowrank_tanh", xptr, _i(_code(x)), ctypes.c_longlong(x.stride(0)),
-         _ptr(w2), _i(_code(w2)), _ptr(bias), _ptr(out), _i(n), _i(low), _i(m), _stream())
+         _ptr(w2), _i(_code(w2)), _ptr(bias), _ptr(out), _i(n), _i(low), _i(m), _i(1 if tanh else 0), _stream())
     return out
 
 
@@ -1173,6 +1287,76 @@ def general_delta(x: torch.Tensor, r_column: int, k_column: int, v_column: int, 
          _i(r_column), _i(k_column), _i(v_column), _i(a_column), _ptr(decay_logits), _ptr(a_bias), sp, ss, _ptr(entry_start),
          _ptr(slots), _ptr(out), _i(entry_start.numel() - 1), _i(n_heads), _i(key_dim), _i(value_dim), _f(decay_scale),
          _f(key_eps), _stream())
+    return out
+
+
+def delta_rule_channel(qkv: torch.Tensor, beta: torch.Tensor, beta_column: int, decay_logits: torch.Tensor,
+                       a_log: torch.Tensor, state: torch.Tensor, entry_start: torch.Tensor, slots: torch.Tensor,
+                       out: torch.Tensor, n_heads: int, n_kv: int, key_dim: int, value_dim: int) -> torch.Tensor:
+    """The gated delta rule with a decay per key channel, S <- diag(g) S with g = exp(-exp(a_log[h]) softplus(z)), over
+    the tokens of every entry, from and into state[slot] ([H, Dv, D] float32).  qkv as for delta_rule; beta: a 2-d
+    tensor whose rows are the tokens', with the H logits of the write strength from column beta_column; decay_logits
+    z [n, H * D] float32; out [n, H * Dv] float32."""
+    n = qkv.shape[0]
+    c = 2 * n_kv * key_dim + n_heads * value_dim
+    _chk(qkv, "delta_rule_channel.qkv", None, (n, c))
+    _chk(beta, "delta_rule_channel.beta")
+    if beta.dim() != 2 or beta.shape[0] != n or beta.shape[1] < beta_column + n_heads:
+        raise KernelError(f"delta_rule_channel.beta: shape {tuple(beta.shape)} has no {n_heads} columns from {beta_column}")
+    if beta.dtype != torch.float32 and beta.dtype != qkv.dtype:
+        raise KernelError(f"delta_rule_channel: logits of dtype {beta.dtype} beside inputs of {qkv.dtype}")
+    _chk(decay_logits, "delta_rule_channel.decay_logits", torch.float32, (n, n_heads * key_dim))
+    _chk(a_log, "delta_rule_channel.a_log", torch.float32, (n_heads,))
+    _chk(out, "delta_rule_channel.out", torch.float32, (n, n_heads * value_dim))
+    _chk(entry_start, "delta_rule_channel.entry_start", torch.int32)
+    _chk(slots, "delta_rule_channel.slots", torch.int32)
+    if not 1 <= key_dim <= DELTA_MAX_KEY_DIM or n_heads % n_kv:
+        raise KernelError(f"delta_rule_channel: heads {n_heads}/{n_kv} of {key_dim}")
+    sp, ss = _state_rows(state, "delta_rule_channel", n_heads * key_dim * value_dim)
+    bptr = ctypes.c_void_p(beta.data_ptr() + beta_column * beta.element_size())
+    _run(load_lib("vt_delta", half=_half(qkv, beta)), "vt_delta_rule_channel", _ptr(qkv), _i(_code(qkv)), bptr, _i(_code(beta)),
+         ctypes.c_longlong(beta.stride(0)), _ptr(decay_logits), _ptr(a_log), sp, ss, _ptr(entry_start), _ptr(slots),
+         _ptr(out), _i(entry_start.numel() - 1), _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _stream())
+    return out
+
+
+def matrix_memory_state_floats(n_heads: int, key_dim: int, value_dim: int) -> int:
+    """Floats of a request's state for matrix_memory: the heads' matrices [H, Dv, D], then per head and block of 16
+    value columns a normalizer [D], then per head and block the running maximum."""
+    zb = -(-value_dim // 16)
+    return n_heads * value_dim * key_dim + n_heads * zb * key_dim + n_heads * zb
+
+
+def matrix_memory(x: torch.Tensor, q_column: int, k_column: int, v_column: int, i_column: int, f_column: int,
+                  i_bias: Optional[torch.Tensor], f_bias: Optional[torch.Tensor], state: torch.Tensor,
+                  entry_start: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, n_heads: int, key_dim: int,
+                  value_dim: int, gate_cap: float, q_scale: float) -> torch.Tensor:
+    """The matrix memory of xLSTM over the tokens of every entry, from and into state[slot] (float32,
+    matrix_memory_state_floats long, zero at the start of a sequence).  With i = cap tanh((a_i + i_bias) / cap) and
+    f = logsigmoid(cap tanh((a_f + f_bias) / cap)) (cap 0: no cap):
+        m' = max(f + m, i);  S <- e^(f + m - m') S + e^(i - m') k v^T;  n <- e^(f + m - m') n + e^(i - m') k;
+        o = S^T (q_scale q) / (max(|n . q_scale q|, e^(-m')) + 1e-6).
+    x: a 2-d tensor whose rows are the tokens', with H heads of D queries from q_column, of D keys from k_column, of
+    Dv values from v_column, and the H logits a_i from i_column and a_f from f_column; out [n, H * Dv] float32."""
+    n = x.shape[0]
+    hd = n_heads * key_dim
+    _chk(x, "matrix_memory.x")
+    if x.dim() != 2 or min(q_column, k_column, v_column, i_column, f_column) < 0 or \
+            x.shape[1] < max(max(q_column, k_column) + hd, v_column + n_heads * value_dim, max(i_column, f_column) + n_heads):
+        raise KernelError(f"matrix_memory.x: shape {tuple(x.shape)} does not hold its columns")
+    for b, name in ((i_bias, "i_bias"), (f_bias, "f_bias")):
+        if b is not None:
+            _chk(b, "matrix_memory." + name, torch.float32, (n_heads,))
+    _chk(out, "matrix_memory.out", torch.float32, (n, n_heads * value_dim))
+    _chk(entry_start, "matrix_memory.entry_start", torch.int32)
+    _chk(slots, "matrix_memory.slots", torch.int32)
+    if not 1 <= key_dim <= DELTA_MAX_KEY_DIM or gate_cap < 0:
+        raise KernelError(f"matrix_memory: keys of {key_dim} (up to {DELTA_MAX_KEY_DIM}), cap {gate_cap}")
+    sp, ss = _state_rows(state, "matrix_memory", matrix_memory_state_floats(n_heads, key_dim, value_dim))
+    _run(load_lib("vt_delta", half=_half(x)), "vt_matrix_memory", _ptr(x), _i(_code(x)), ctypes.c_longlong(x.stride(0)),
+         _i(q_column), _i(k_column), _i(v_column), _i(i_column), _i(f_column), _ptr(i_bias), _ptr(f_bias), sp, ss,
+         _ptr(entry_start), _ptr(slots), _ptr(out), _i(entry_start.numel() - 1), _i(n_heads), _i(key_dim), _i(value_dim),
+         _f(gate_cap), _f(q_scale), _stream())
     return out
 
 

@@ -14,8 +14,18 @@ import torch
 
 from ..config.base import LayerSpec, ModelSpec, PartSpec
 from ..kernels import ops
+from ..parts.linear import linear
 from ..parts.base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, NormedInput, Part, Registry,
                           Runtime, TensorDecl)
+
+
+def settle(h: torch.Tensor, delta):
+    """Adds what a layer has handed on unadded (a tensor, a pair of tensors, or nothing) to the stream."""
+    if isinstance(delta, tuple):
+        return ops.residual_add2(h, delta[0], delta[1])
+    if isinstance(delta, torch.Tensor):
+        return ops.residual_add(h, delta)
+    return h
 
 
 def build_part(registry: Registry, spec: PartSpec, prefix: str, **context):
@@ -41,6 +51,9 @@ class DecoderModel:
         self.offsets_name: Optional[str] = spec.stream_offsets["name"] if spec.stream_offsets else None
         self.offsets_rows = int(spec.stream_offsets["rows"]) if spec.stream_offsets else 0
         self.offsets: Optional[torch.Tensor] = None
+        # the matrix W [width, 2 width] of x <- W [x; x0] in front of the schedule entries that say `inject`
+        self.inject_name: Optional[str] = spec.stream_inject["name"] if spec.stream_inject else None
+        self.w_inject = self.p_inject = None
         # several residual streams: [tokens, streams, width] between the embedding and the final norm
         self.streams = int(spec.streams)
         self._stream_ones: Optional[torch.Tensor] = None
@@ -70,6 +83,8 @@ class DecoderModel:
                     out[name] = decl
         if self.offsets_name:
             out[self.offsets_name] = TensorDecl((self.offsets_rows, self.spec.hidden_size), "bias")
+        if self.inject_name:
+            out[self.inject_name] = TensorDecl((self.spec.hidden_size, 2 * self.spec.hidden_size), "matrix")
         return out
 
     def load(self, get: Callable[[str], torch.Tensor]) -> None:
@@ -80,6 +95,10 @@ class DecoderModel:
         self.final_norm.load(get, self.rt)
         if self.offsets_name:
             self.offsets = self.rt.place(get(self.offsets_name), "bias")
+        if self.inject_name:
+            w = self.rt.place(get(self.inject_name), "matrix")
+            self.p_inject = self.rt.pack(w)
+            self.w_inject = self.rt.row_major(w, self.p_inject)
         # a head's loader takes `shared`: tensors by name that other parts have already placed on the device (the
         # embedding's table, which a tied head multiplies by)
         shared = {}
@@ -96,10 +115,25 @@ class DecoderModel:
             # every stream starts as the embedding's output
             h = ops.streams_fill(h, self.rt.buffer("streams", (h.shape[0], self.streams, h.shape[1]), torch.float32))
         delta = None
+        first = None
+        if self.inject_name:
+            # the embedding's output is kept: passes of a repeated run of layers start from it again
+            first = ops.set_plus_row(self.rt.buffer("h.first", tuple(h.shape), torch.float32), h, None)
         last = len(self.schedule) - 1
         for i, entry in enumerate(self.schedule):
             block = self.layers[entry.layer]
-            if entry.offset_row is not None:
+            if isinstance(delta, tuple) and (entry.inject or entry.offset_row is not None
+                                             or not getattr(block, "takes_pair", False)):
+                h, delta = settle(h, delta), None
+            if entry.inject:
+                # x <- W [x; x0] (+ the entry's offset): one product over the joined rows, its result is the new stream
+                h = settle(h, delta)
+                delta = None
+                width = h.shape[1]
+                joined = ops.concat_cast(h, first, self.rt.buffer("h.joined", (h.shape[0], 2 * width), self.rt.dtype))
+                y = linear(self.rt, joined, self.w_inject, None, "h.injected", packed=self.p_inject)
+                ops.set_plus_row(h, y, self.offsets[entry.offset_row] if entry.offset_row is not None else None)
+            elif entry.offset_row is not None:
                 # what is still to be added goes in with the offset, in one pass over the stream
                 ops.add_row(h, delta if isinstance(delta, torch.Tensor) else None, self.offsets[entry.offset_row])
                 delta = None
@@ -108,7 +142,7 @@ class DecoderModel:
                 # the stream still changes in between)
                 behind = self.schedule[i + 1] if i < last else None
                 nxt = (getattr(self.layers[behind.layer], "first_norm", None)
-                       if behind is not None and behind.offset_row is None else None)
+                       if behind is not None and behind.offset_row is None and not behind.inject else None)
                 h, delta = block.forward(h, delta, ctx, caches[i], states[i], next_norm=nxt)
             else:
                 if isinstance(delta, NormedInput):
@@ -118,6 +152,10 @@ class DecoderModel:
             return None
         if isinstance(delta, NormedInput):
             delta = None
+        if isinstance(delta, tuple):
+            if getattr(self.final_norm, "takes_pair", False) and not self.streams:
+                return self.head.forward(self.final_norm.forward(h, delta[0], rows=ctx.logit_rows, delta2=delta[1]))
+            h, delta = settle(h, delta), None
         if self.streams:
             # the streams' sum, for the wanted rows only, inside the final norm's kernel
             if self._stream_ones is None:

@@ -80,6 +80,58 @@ class PreNormBlock(Part):
         return part.forward(x, *args)
 
 
+@BLOCKS.register("parallel")
+class ParallelBlock(Part):
+    """One norm whose output the mixer and the feed-forward both read; their results join the stream in one sum:
+
+        h = norm(x);   x <- x + (mixer(h) + feed_forward(h))
+
+    The block hands both results on unadded (a pair), so that the norm of the layer behind it adds them in the kernel
+    that normalises (a norm with `delta2`); whoever cannot take a pair gets them added first (`settle`).  A layer
+    without a feed-forward hands the mixer's result on alone."""
+
+    norm_roles = ("input",)
+    replayable = True
+    takes_pair = True       # forward(h, delta, ...) with delta a pair of tensors: both are still to be added to h
+
+    def __init__(self, *, rt: Runtime, norms, mixer, feed_forward, prefix: str = "", width: int = 0):
+        self.rt = rt
+        self.norm_in = norms["input"]
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+
+    def parts(self):
+        return [self.norm_in, self.mixer] + ([self.feed_forward] if self.feed_forward is not None else [])
+
+    @staticmethod
+    def settle(h: torch.Tensor, delta):
+        """Adds what is still to be added to the stream (a tensor, a pair of tensors or None); returns h."""
+        if isinstance(delta, tuple):
+            return ops.residual_add2(h, delta[0], delta[1])
+        if isinstance(delta, torch.Tensor):
+            return ops.residual_add(h, delta)
+        return h
+
+    def forward(self, h: torch.Tensor, delta, ctx, cache, state) -> Tuple[torch.Tensor, object]:
+        if isinstance(delta, NormedInput):
+            delta = None            # (its addition is done; this block applies its own norm)
+        if isinstance(delta, tuple) and not getattr(self.norm_in, "takes_pair", False):
+            h, delta = self.settle(h, delta), None
+        if isinstance(delta, tuple):
+            x = self.norm_in.forward(h, delta[0], delta2=delta[1])
+        else:
+            x = self.norm_in.forward(h, delta)
+        y = self.mixer.forward(x, ctx, cache, state)
+        if self.feed_forward is None:
+            return h, y
+        z = self.feed_forward.forward(x, ctx)
+        if y.dtype != z.dtype:
+            # (results of different types are joined in the stream one after the other)
+            ops.residual_add(h, y)
+            return h, z
+        return h, (y, z)
+
+
 @BLOCKS.register("hyper")
 class HyperBlock(Part):
     """Pre-norm sublayers around S residual streams x_1 .. x_S (float32, [tokens, S, width]) instead of one.  For

@@ -14,7 +14,8 @@ biases if the model has them,
     g <- min(g, limit),  u <- clamp(u, -limit, limit)        (limit 0: no bounds)
     act = g * sigmoid(alpha * g * (1 + cubic * g^2)) * (u + up_shift)
 
-alpha 1, no bounds, no shift and cubic 0 is SiLU gating, the reference's.  activation "gelu_tanh" is the tanh form of
+alpha 1, no bounds, no shift and cubic 0 is SiLU gating, the reference's.  activation "relu" is max(g, 0) * (u +
+up_shift), the form's limit for alpha -> infinity, which the kernels compute as such.  activation "gelu_tanh" is the tanh form of
 GELU, 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))): since (1 + tanh z) / 2 = sigmoid(2 z) it is the same form
 with alpha = 2 sqrt(2 / pi) and cubic = 0.044715.
 """
@@ -47,9 +48,13 @@ class GatedMLP(Part):
             if act_alpha != 1.0 or act_cubic != 0.0:
                 raise ValueError("activation 'gelu_tanh' fixes act_alpha and act_cubic")
             act_alpha, act_cubic = 2.0 * math.sqrt(2.0 / math.pi), 0.044715
+        elif activation == "relu":
+            if act_alpha != 1.0 or act_cubic != 0.0:
+                raise ValueError("activation 'relu' fixes act_alpha and act_cubic")
+            act_alpha = math.inf        # the sigmoid of the gate's form as a step (the kernels test for it)
         elif activation != "silu":
             raise ValueError(f"activation '{activation}' is not supported ('silu', whose form act_alpha, act_limit, "
-                             f"up_shift and act_cubic change, and 'gelu_tanh' are)")
+                             f"up_shift and act_cubic change, 'gelu_tanh' and 'relu' are)")
         if not act_alpha > 0 or act_limit < 0:
             raise ValueError("act_alpha must be positive and act_limit not negative (0: no bounds)")
         self.alpha, self.limit, self.shift, self.cubic = float(act_alpha), float(act_limit), float(up_shift), float(act_cubic)

@@ -4,8 +4,12 @@ keys scaled to unit root mean square, queries that grow with the logarithm of
 the position, scores capped by a tanh or lowered by a slope times the
 distance, keys masked by a window or by chunks of positions, a learned sink in
 the softmax's denominator, values mixed with those of an earlier layer, and
-one sigmoid gate per head on the output.  Every one of these is a constructor
-parameter that can be left out.
+one sigmoid gate per head (or per element) on the output, a gain on the
+unit-RMS queries and keys, a bias that grows with the logarithm of the
+distance, a learned shift of every score per head, weights that are sigmoids of
+the scores instead of a softmax, neighbouring elements rotated together, a bias
+on the output projection.  Every one of these is a constructor parameter that
+can be left out.
 
 Per token: q, k, v (and the gates' logits) in one matrix product with the
 biases; rotation, unit scaling and the write into the pages in one kernel;
@@ -18,6 +22,12 @@ reads the pages; output projection.
     j is seen from i  <=>  j <= i,  i - j < window (if window > 0),  floor(j / chunk) = floor(i / chunk) (if chunk > 0)
     p_ij = exp(score(i, j)) / (sum_j' exp(score(i, j')) + exp(sink_h))                        (no sink: the plain softmax)
     out_i[h] = sigmoid(gate_i[h]) * sum_j p_ij v_j
+
+    distance_log:  score(i, j) -= r1_h * ln(1 + r2_h * (i - j))        r1, r2 learned, one each per head
+    score_shift:   score(i, j) += shift_h                              learned, one per head
+    weights "sigmoid":  p_ij = sigmoid(score(i, j)) for every seen j, not normalized (no sink)
+    out_gate:      out_i[h][d] *= sigmoid((W_g x_i)[h][d])             one logit per output element instead of per head
+    qk_gain:       after the unit-RMS scaling q and k are multiplied by a learned gain per element (shared by heads)
 
 Value mixing ties layers together: the first layer of a model that says value_mix="source" leaves the step's values
 in a buffer, and every layer that says value_mix="mix" keeps (1 - lambda) v + lambda v_source in its pages instead
@@ -61,13 +71,15 @@ def plan_tiles(ctx) -> Optional[Dict[tuple, np.ndarray]]:
 
 def run_masked_attention(rt: Runtime, ctx, cache, q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, d: int, dv: int,
                          scale: float, softcap: float = 0.0, window: int = 0, chunk: int = 0, gate=None,
-                         gate_column: int = 0, sink=None, slopes=None) -> torch.Tensor:
+                         gate_column: int = 0, sink=None, slopes=None, dist_log=None, score_shift=None,
+                         sigmoid_weights: bool = False, gate_wide: bool = False) -> torch.Tensor:
     """The attention itself over a layer's pages, by the kernel that suits the step: in the 16-bit types with heads
     in multiples of 16, steps of single tokens go to the matrix-core kernel whose rows are the heads of a key/value
     group and whose keys are dealt out to many waves, steps with portions of prompts to the one whose rows are tokens
     (tiles planned by `plan_tiles`); everything else, and float32 always, to the kernel with a block per (token, head)."""
     cores = rt.lowp and ops.attention_masked_mfma_takes(d, dv, cache["k"].shape[2])
-    kw = dict(gate=gate, gate_column=gate_column, sink=sink, slopes=slopes)
+    kw = dict(gate=gate, gate_column=gate_column, sink=sink, slopes=slopes, dist_log=dist_log, score_shift=score_shift,
+              sigmoid_weights=sigmoid_weights, gate_wide=gate_wide)
     if cores and ctx.single_token:
         n = q.shape[0]
         splits = ops.attention_masked_decode_splits(n, nh, nkv, ctx.n_positions)
@@ -96,7 +108,9 @@ class MaskedAttention(Part):
                  scale: Optional[float] = None, softcap: float = 0.0, window: int = 0, chunk: int = 0,
                  unit_rms_eps: Optional[float] = None, head_gate: bool = False, shared: Optional[dict] = None,
                  names: Optional[Dict[str, str]] = None, sink: bool = False, distance_slopes: Optional[float] = None,
-                 q_temp: Optional[Dict[str, float]] = None, value_mix: Optional[str] = None, fuse_norms: bool = False):
+                 q_temp: Optional[Dict[str, float]] = None, value_mix: Optional[str] = None, fuse_norms: bool = False,
+                 rot_pairs: str = "halves", qk_gain: bool = False, distance_log: bool = False, score_shift: bool = False,
+                 weights: str = "softmax", out_gate: bool = False, o_bias: bool = False):
         """key_dim / value_dim: sizes of a head's queries and keys / of its values (default: the same);
         position: a rotary encoding whose `dim` may be smaller than key_dim (the rest of a head passes unchanged);
         unit_rms_eps: queries and keys are divided by their root mean square per head after the rotation, with
@@ -110,7 +124,13 @@ class MaskedAttention(Part):
         None; fuse_norms: with
         few rows in bfloat16 the input product applies the norm in front of the mixer and the output product adds to
         the residual stream and prepares the norm behind (as `PagedAttention` does; it rounds the stream times the
-        norm's gains to 16 bits before the division by the root instead of after it)."""
+        norm's gains to 16 bits before the division by the root instead of after it);
+        rot_pairs: "halves" (element i turns with element i + dims/2) or "neighbours" (element 2i with 2i + 1: the
+        rows of W_q and W_k and their biases are reordered when they are loaded, after which the kernels' half-split
+        rotation is the neighbouring one, and a score, a sum over the elements of q and k alike, does not see the
+        order); qk_gain (with unit_rms_eps): tensors q_norm, k_norm [key_dim]; distance_log: tensors r1, r2 [heads];
+        score_shift: tensor shift [heads]; weights: "softmax" or "sigmoid"; out_gate: an elementwise sigmoid gate from
+        a projection g [heads * value_dim, width] (head_gate's tensor name; not both); o_bias: tensor o_bias [width]."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
         self.rt, self.width = rt, int(width)
@@ -137,10 +157,27 @@ class MaskedAttention(Part):
         if value_mix not in (None, "off", "source", "mix"):
             raise ValueError(f"value_mix {value_mix!r} ('source', 'mix', 'off' or None)")
         self.value_mix = value_mix
+        if rot_pairs not in ("halves", "neighbours"):
+            raise ValueError(f"rot_pairs {rot_pairs!r} ('halves' or 'neighbours')")
+        if weights not in ("softmax", "sigmoid"):
+            raise ValueError(f"weights {weights!r} ('softmax' or 'sigmoid')")
+        self.rot_pairs, self.sigmoid_weights = rot_pairs, weights == "sigmoid"
+        self.qk_gain, self.distance_log, self.score_shift = bool(qk_gain), bool(distance_log), bool(score_shift)
+        self.out_gate, self.o_bias = bool(out_gate), bool(o_bias)
+        if self.qk_gain and self.unit_rms_eps is None:
+            raise ValueError("qk_gain is a gain on unit-RMS queries and keys: give unit_rms_eps")
+        if self.qk_gain and rot_pairs == "neighbours" and position is not None:
+            raise ValueError("a gain per element and reordered rotated elements are not combined")
+        if self.out_gate and self.head_gate:
+            raise ValueError("one gate on the output: per head or per element")
+        if self.sigmoid_weights and self.has_sink:
+            raise ValueError("sigmoid weights have no denominator for a sink to join")
         # what the block asks for (parts/block.py)
         self.takes_normed_input = self.hands_norm_on = bool(fuse_norms)
         n = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "g": "g_proj.weight",
-             "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "sink": "sink", "vmix": "vmix"}
+             "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "sink": "sink", "vmix": "vmix",
+             "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "r1": "r1", "r2": "r2", "shift": "shift",
+             "o_bias": "o_proj.bias"}
         n.update(names or {})
         self.names = {k: prefix + v for k, v in n.items()}
         pos_spec = position or PartSpec("none", {})
@@ -155,6 +192,7 @@ class MaskedAttention(Part):
             raise ValueError("this mixer takes rotary position encodings (or none)")
         self.w_in = self.b_in = self.b_in_lowp = self.p_in = self.w_o = self.p_o = None
         self.sink = self.slopes = self.v_lambda = None
+        self.q_gain = self.k_gain = self.r1 = self.r2 = self.shift = self.b_o = self.b_o_lowp = None
 
     # columns of the input projection: queries, keys, values, gates
     @property
@@ -198,6 +236,18 @@ class MaskedAttention(Part):
             t[nm["v_bias"]] = TensorDecl((self.nkv * self.dv,), "bias")
         if self.head_gate:
             t[nm["g"]] = TensorDecl((self.nh, self.width), "matrix")
+        if self.out_gate:
+            t[nm["g"]] = TensorDecl((self.nh * self.dv, self.width), "matrix")
+        if self.qk_gain:
+            t[nm["q_norm"]] = TensorDecl((self.d,), "gain")
+            t[nm["k_norm"]] = TensorDecl((self.d,), "gain")
+        if self.distance_log:
+            t[nm["r1"]] = TensorDecl((self.nh,), "bias")
+            t[nm["r2"]] = TensorDecl((self.nh,), "bias")
+        if self.score_shift:
+            t[nm["shift"]] = TensorDecl((self.nh,), "bias")
+        if self.o_bias:
+            t[nm["o_bias"]] = TensorDecl((self.width,), "bias")
         if self.has_sink:
             t[nm["sink"]] = TensorDecl((self.nh,), "bias")
         if self.value_mix is not None:
@@ -205,16 +255,39 @@ class MaskedAttention(Part):
             t[nm["vmix"]] = TensorDecl((), "bias", optional=self.value_mix != "mix")
         return t
 
+    def _pair_order(self, t: torch.Tensor, heads: int) -> torch.Tensor:
+        """Rows (or elements) of the heads of a query or key projection in the order in which the kernels' half-split
+        rotation is the neighbouring one: of a head's first `dims` elements, element 2i goes to place i and element
+        2i + 1 to place i + dims/2."""
+        dims = int(getattr(self.position, "dim", 0))
+        if self.rot_pairs != "neighbours" or dims == 0:
+            return t
+        order = torch.cat([torch.arange(0, dims, 2), torch.arange(1, dims, 2), torch.arange(dims, self.d)])
+        index = (torch.arange(heads)[:, None] * self.d + order[None, :]).reshape(-1).to(t.device)
+        return t.index_select(0, index)
+
     def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
         nm = self.names
-        mats = [rt.place(get(nm[k]), "matrix") for k in (("q", "k", "v", "g") if self.head_gate else ("q", "k", "v"))]
+        gated = self.head_gate or self.out_gate
+        mats = [rt.place(get(nm[k]), "matrix") for k in (("q", "k", "v", "g") if gated else ("q", "k", "v"))]
+        mats[0], mats[1] = self._pair_order(mats[0], self.nh), self._pair_order(mats[1], self.nkv)
         self.w_in = torch.cat(mats, dim=0).contiguous()
         if self.qkv_bias:
             b = [rt.place(get(nm[k]), "bias") for k in ("q_bias", "k_bias", "v_bias")]
-            if self.head_gate:
-                b.append(torch.zeros(self.nh, dtype=torch.float32, device=rt.device))
+            b[0], b[1] = self._pair_order(b[0], self.nh), self._pair_order(b[1], self.nkv)
+            if gated:
+                b.append(torch.zeros(mats[3].shape[0], dtype=torch.float32, device=rt.device))
             self.b_in = torch.cat(b, dim=0).contiguous()
             self.b_in_lowp = self.b_in.to(rt.dtype)
+        if self.qk_gain:
+            self.q_gain, self.k_gain = rt.place(get(nm["q_norm"]), "gain"), rt.place(get(nm["k_norm"]), "gain")
+        if self.distance_log:
+            self.r1, self.r2 = rt.place(get(nm["r1"]), "bias"), rt.place(get(nm["r2"]), "bias")
+        if self.score_shift:
+            self.shift = rt.place(get(nm["shift"]), "bias")
+        if self.o_bias:
+            self.b_o = rt.place(get(nm["o_bias"]), "bias")
+            self.b_o_lowp = self.b_o.to(rt.dtype)
         self.w_o = rt.place(get(nm["o"]), "matrix")
         if self.has_sink:
             self.sink = rt.place(get(nm["sink"]), "bias")
@@ -241,9 +314,12 @@ class MaskedAttention(Part):
         # the values that layers mix: one buffer per model and step, written by the source layer, read by the others
         v_first = rt.buffer("mattn.v_first", (n, nkv * dv), torch.float32) if self.value_mix in ("source", "mix") else None
         ops.qk_prepare(y, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache["k"], cache["v"], nh, nkv,
-                       d, dv, self.unit_rms_eps, q_temp=self.q_temp, v_first=v_first, v_lambda=self.v_lambda)
+                       d, dv, self.unit_rms_eps, q_temp=self.q_temp, v_first=v_first, v_lambda=self.v_lambda,
+                       q_gain=self.q_gain, k_gain=self.k_gain)
         out = rt.buffer("mattn.out", (n, nh * dv), rt.dtype)
         run_masked_attention(rt, ctx, cache, q, out, nh, nkv, d, dv, self.scale, self.softcap, self.window, self.chunk,
-                             gate=y if self.head_gate else None, gate_column=self._gate_column, sink=self.sink,
-                             slopes=self.slopes)
-        return linear(rt, out, self.w_o, None, "mattn.o", packed=self.p_o, residual=residual, hand_on=hand_on)
+                             gate=y if (self.head_gate or self.out_gate) else None, gate_column=self._gate_column,
+                             sink=self.sink, slopes=self.slopes, dist_log=(self.r1, self.r2) if self.distance_log else None,
+                             score_shift=self.shift, sigmoid_weights=self.sigmoid_weights, gate_wide=self.out_gate)
+        return linear(rt, out, self.w_o, self.b_o, "mattn.o", bias_lowp=self.b_o_lowp, packed=self.p_o, residual=residual,
+                      hand_on=hand_on)

@@ -55,3 +55,42 @@ class RMSNorm(Part):
         n = rows.numel() if rows is not None else h.shape[0]
         out = self.rt.buffer(self.scratch + (".rows" if rows is not None else ""), (n, self.width), self.rt.dtype)
         return ops.rmsnorm(h, delta, self.gain, out, self.eps, rows=rows)
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Part):
+    """Layer norm with a gain and (optionally) a bias: out = (x - mean) / sqrt(var + eps) * gain + bias, the variance
+    the mean of the squared deviations, all in float32, fused with the residual additions in front of it.  Beside
+    `delta` it takes `delta2`: with both, x = h + (delta + delta2), the sum of two sublayers that ran side by side."""
+
+    replayable = True
+    takes_pair = True       # forward(h, delta, delta2=): two addends of one type in front of the norm
+
+    def __init__(self, *, rt: Runtime, width: int, prefix: str, eps: float, name: str = "weight", bias_name: Optional[str] = None,
+                 scratch: str = "norm"):
+        """name / bias_name: the tensors' names behind the prefix (bias_name None: no bias)."""
+        self.rt = rt
+        self.width = int(width)
+        self.eps = float(eps)
+        self.name = prefix + name
+        self.bias_name = prefix + bias_name if bias_name is not None else None
+        self.scratch = scratch
+        self.gain: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        t = {self.name: TensorDecl((self.width,), "gain")}
+        if self.bias_name is not None:
+            t[self.bias_name] = TensorDecl((self.width,), "bias")
+        return t
+
+    def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
+        self.gain = rt.place(get(self.name), "gain")
+        if self.bias_name is not None:
+            self.bias = rt.place(get(self.bias_name), "bias")
+
+    def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+                delta2: Optional[torch.Tensor] = None) -> torch.Tensor:
+        n = rows.numel() if rows is not None else h.shape[0]
+        out = self.rt.buffer(self.scratch + (".rows" if rows is not None else ""), (n, self.width), self.rt.dtype)
+        return ops.layernorm(h, delta, self.gain, self.bias, out, self.eps, rows=rows, delta2=delta2)
