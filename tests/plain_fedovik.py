@@ -227,9 +227,13 @@ def mixer(L: dict, h, w, p: str, eps: float, pos) -> torch.Tensor:
     raise ValueError(L["type"])
 
 
-def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], streams: Optional[list] = None) -> torch.Tensor:
+def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], streams: Optional[list] = None,
+            rounded: bool = False) -> torch.Tensor:
     """Logits [T, vocab] of one sequence from position 0.  streams: a list that gets the residual stream after every
-    layer run."""
+    layer run.  rounded: what the sublayers and the re-entry read is rounded to bfloat16 first, everything else stays
+    float64: how far rounding alone moves the logits of this model."""
+    def r16(t):
+        return t.to(torch.bfloat16).to(DT) if rounded else t
     w = {k: v.to(DT) for k, v in w.items()}
     eps = cfg["norm"]["eps"]
     pos = torch.arange(len(ids))
@@ -237,16 +241,16 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], streams: Opti
     x = x0
     for i, t in layer_runs(cfg):
         if t is not None:
-            x = torch.cat([x, x0], dim=-1) @ w["loop.in"].t() + w["loop.step"][t]
+            x = r16(torch.cat([x, x0], dim=-1)) @ w["loop.in"].t() + w["loop.step"][t]
         L, p = cfg["layers"][i], f"l{i}."
-        h = layer_norm(x, w[p + "norm1"], w[p + "norm1.b"], eps)
+        h = r16(layer_norm(x, w[p + "norm1"], w[p + "norm1.b"], eps))
         y = mixer(L, h, w, p + "mix.", eps, pos)
         if L.get("mlp"):
             y = y + relu_mlp(h, w, p + "mlp.")
         x = x + y
         if streams is not None:
             streams.append(x.clone())
-    return layer_norm(x, w["final.norm"], w["final.norm.b"], eps) @ w["embed"].t()
+    return r16(layer_norm(x, w["final.norm"], w["final.norm.b"], eps)) @ w["embed"].t()
 
 
 def greedy(cfg: dict, w: Dict[str, torch.Tensor], prompt: List[int], n_new: int) -> List[int]:

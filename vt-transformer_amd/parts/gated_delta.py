@@ -100,27 +100,27 @@ class GatedDeltaMixer(Part):
 
     def tensors(self) -> Dict[str, TensorDecl]:
         nm, kd, vd = self.names, self.nkv * self.d, self.nh * self.dv
+        # (the order of a dict is the order in which a model's tensors are listed and drawn)
         t = {
             nm["q"]: TensorDecl((kd, self.width), "matrix"),
             nm["k"]: TensorDecl((kd, self.width), "matrix"),
             nm["v"]: TensorDecl((vd, self.width), "matrix"),
-            nm["o"]: TensorDecl((self.width, vd), "matrix"),
-            nm["b"]: TensorDecl((self.nh, self.width), "matrix"),
-            nm["A_log"]: TensorDecl((self.nh,), "bias"),
-            nm["norm"]: TensorDecl((self.dv,), "gain"),
         }
         if self.gate_rank:
             t[nm["g1"]] = TensorDecl((self.gate_rank, self.width), "matrix")
             t[nm["g2"]] = TensorDecl((vd, self.gate_rank), "matrix")
         else:
             t[nm["g"]] = TensorDecl((vd, self.width), "matrix")
+        t[nm["o"]] = TensorDecl((self.width, vd), "matrix")
+        t[nm["b"]] = TensorDecl((self.nh, self.width), "matrix")
         if self.channel_decay:
             t[nm["a1"]] = TensorDecl((self.decay_rank, self.width), "matrix")
             t[nm["a2"]] = TensorDecl((self.nh * self.d, self.decay_rank), "matrix")
-            t[nm["dt_bias"]] = TensorDecl((self.nh * self.d,), "bias")
         else:
             t[nm["a"]] = TensorDecl((self.nh, self.width), "matrix")
-            t[nm["dt_bias"]] = TensorDecl((self.nh,), "bias")
+        t[nm["A_log"]] = TensorDecl((self.nh,), "bias")
+        t[nm["dt_bias"]] = TensorDecl((self.nh * self.d if self.channel_decay else self.nh,), "bias")
+        t[nm["norm"]] = TensorDecl((self.dv,), "gain")
         # (with one tap the "convolution" is a factor per channel: the tensors are there all the same)
         t[nm["q_conv"]] = TensorDecl((kd, self.taps), "bias")
         t[nm["k_conv"]] = TensorDecl((kd, self.taps), "bias")
