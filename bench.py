@@ -234,6 +234,26 @@ def kigalix_pair_configs(key: str, streams: int):
     return kig, gab
 
 
+def fedovik_pair_configs(key: str, window: int):
+    """(Fedovik config.json, Lisunex config.json) of equal sizes.  Fedovik: sigmoid attention, the pair of windowed
+    attention and channel-decay delta rule, and the matrix memory in turn, each beside a ReLU feed-forward under one
+    layer norm; the pair's attention sees `window` positions, its delta rule and the matrix memory have Lisunex's heads.  Lisunex: the pair of `pair_configs` with chunks of `window` positions."""
+    width, layers, heads, kv, d, ff, vocab = PAIR_SIZES[key]
+    mlp = {"kind": "dense", "ff": ff}
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "rot": {"dims": d // 2, "base": 1e6}}}
+    pair = {"type": "parallel", "mlp": mlp,
+            "mixer": {"left": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": window}},
+                      "right": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "conv": 4,
+                                "a_rank": 64, "g_rank": 64},
+                      "left_scale": 1.0, "right_scale": 1.0}}
+    mem = {"type": "mlstm", "mlp": mlp, "mixer": {"heads": heads, "dim": d, "vdim": d, "gate_cap": 15.0}}
+    fed = {"architecture": "Fedovik", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6},
+           "layers": [(att, pair, mem)[i % 3] for i in range(layers)], "loop": None, "max_positions": 32768}
+    lis, _ = pair_configs(key, window)
+    return fed, lis
+
+
 class PairBench(Bench):
     """Bench's measurements on an engine built from any config.json."""
 
@@ -256,10 +276,10 @@ class PairBench(Bench):
 
 
 def design_pairs(args, design: str) -> int:
-    """Prefill and decode of a second design (lisunex or gabelorn beside Qwen2, kigalix beside Gabelorn) at equal
-    sizes; one JSON line."""
+    """Prefill and decode of a second design (lisunex or gabelorn beside Qwen2, kigalix beside Gabelorn, fedovik beside
+    Lisunex) at equal sizes; one JSON line."""
     title = design.capitalize()
-    beside = "gabelorn" if design == "kigalix" else "qwen2"
+    beside = {"kigalix": "gabelorn", "fedovik": "lisunex"}.get(design, "qwen2")
     keys = [k.strip() for k in getattr(args, design).split(",") if k.strip()]
     for k in keys:
         if k not in PAIR_SIZES:
@@ -268,8 +288,10 @@ def design_pairs(args, design: str) -> int:
     T, batch, prompt_len = args.prefill_tokens, args.batch, args.prompt_len or 1024
     per_req = -(-(prompt_len + args.steps + args.warmup + 32) // 16) * 16
     pool = max(batch * per_req, T + 64)
-    span = {"lisunex": args.lisunex_chunk, "gabelorn": args.gabelorn_window, "kigalix": args.kigalix_streams}[design]
-    make = {"lisunex": pair_configs, "gabelorn": gabelorn_pair_configs, "kigalix": kigalix_pair_configs}[design]
+    span = {"lisunex": args.lisunex_chunk, "gabelorn": args.gabelorn_window, "kigalix": args.kigalix_streams,
+            "fedovik": args.fedovik_window}[design]
+    make = {"lisunex": pair_configs, "gabelorn": gabelorn_pair_configs, "kigalix": kigalix_pair_configs,
+            "fedovik": fedovik_pair_configs}[design]
     only = getattr(args, "only", "")
     out = {}
     for k in keys:
@@ -301,7 +323,7 @@ def design_pairs(args, design: str) -> int:
         "vs_baseline": None, "dtype": {"bfloat16": "bf16", "float16": "fp16"}[args.dtype],
         "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
         "config": {"model": f"{title} and {beside.capitalize()} at equal sizes", "global_batch": batch, "seq_len": prompt_len,
-                   "prefill_tokens": T, {"lisunex": "chunk", "gabelorn": "window", "kigalix": "streams"}[design]: span,
+                   "prefill_tokens": T, {"lisunex": "chunk", "gabelorn": "window", "kigalix": "streams", "fedovik": "window"}[design]: span,
                    "parallelism": "1 GPU"},
         "pairs": out}), flush=True)
     return 0
@@ -361,17 +383,25 @@ def main() -> int:
                          "sizes, prefill of --prefill-tokens and decode at --batch; sizes by name, with commas: "
                          + ", ".join(PAIR_SIZES))
     ap.add_argument("--kigalix-streams", type=int, default=4, help="residual streams of the Kigalix model")
+    ap.add_argument("--fedovik", default="", metavar="SIZES",
+                    help="another workload instead: the Fedovik design (sigmoid attention, windowed attention beside a "
+                         "channel-decay delta rule, and matrix memory in turn, each beside a ReLU feed-forward) beside "
+                         "Lisunex at equal sizes, prefill of --prefill-tokens and decode at --batch; sizes by name, with "
+                         "commas: " + ", ".join(PAIR_SIZES))
+    ap.add_argument("--fedovik-window", type=int, default=1024, help="positions that the windowed attention of Fedovik sees")
     ap.add_argument("--only", default="", metavar="MODEL",
-                    help="with --lisunex, --gabelorn or --kigalix: measure one model of the pair alone (profiling runs)")
+                    help="with --lisunex, --gabelorn, --kigalix or --fedovik: measure one model of the pair alone "
+                         "(profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; N > 1 is not measured")
         return 2
 
-    if args.lisunex or args.gabelorn or args.kigalix:
+    if args.lisunex or args.gabelorn or args.kigalix or args.fedovik:
         if args.dtype == "float16":
             args.dtype = "bfloat16"         # the serving dtype of these designs
-        return design_pairs(args, "lisunex" if args.lisunex else "gabelorn" if args.gabelorn else "kigalix")
+        return design_pairs(args, "lisunex" if args.lisunex else "gabelorn" if args.gabelorn else
+                            "kigalix" if args.kigalix else "fedovik")
 
     import torch
 

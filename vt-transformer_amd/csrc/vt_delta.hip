@@ -22,12 +22,14 @@
 //     S <- diag(w) S - (a * u)(u^T S) + k v^T,  u = k / sqrt(|k|^2 + eps);   o = S^T r      (both terms read the old S)
 // with w = exp(-c * sigmoid(z)) from decay logits z and a = sigmoid(removal logits), all in float32.
 //   vt_lowrank_tanh:      z[t][j] = bias[j] + sum_l W2[j][l] tanh(x[t][l]): the decay logits from a low-rank projection
-//                         (act 0: without the tanh, for low-rank projections whose middle is linear).
+//                         (act 0: without the tanh, for low-rank projections whose middle is linear; with `a_log` the
+//                         sums leave as decays, exp(-exp(a_log[head]) softplus(sum)): what a recurrence would otherwise
+//                         work out token by token is computed here for all tokens at once).
 //   vt_general_delta:     the recurrence, in vt_delta_rule's arrangement (a row of 16 lanes per state column).
 //
 // The gated delta rule with a decay per key channel (vt_delta_rule_channel): the first rule above with
 //     S <- diag(g) S,   g[d] = exp(-exp(A_log[head]) softplus(z[d]))
-// from decay logits z [n][H * D] in float32 (their bias already added).
+// with the decays g [n][H * D] in float32 computed in front of it (vt_lowrank_tanh with a_log).
 //
 // The matrix memory of xLSTM (vt_matrix_memory): per head S [D][Dv], a normalizer n [D] and a running maximum m of
 // the gates' logarithms, all float32 and all zero at the start of a sequence:
@@ -411,7 +413,7 @@ extern "C" int vt_gated_rmsnorm(const float* o, const float* w, const void* gate
 template <typename TI, typename TW>
 __global__ __launch_bounds__(256) void lowrank_tanh_kernel(const TI* __restrict__ x, long long ldx, const TW* __restrict__ w2,
                                                            const float* __restrict__ bias, float* __restrict__ z, int L, int M,
-                                                           int act) {
+                                                           int act, const float* __restrict__ a_log, int per_head) {
     extern __shared__ float th[];
     const int t = blockIdx.x;
     for (int l = threadIdx.x; l < L; l += 256) {
@@ -423,23 +425,27 @@ __global__ __launch_bounds__(256) void lowrank_tanh_kernel(const TI* __restrict_
     if (j >= M) return;
     float acc = bias ? bias[j] : 0.f;
     for (int l = 0; l < L; ++l) acc = fmaf(load_f32<TW>(w2, (size_t)j * L + l), th[l], acc);
+    // the sums as decay logits: out = exp(-exp(a_log[head]) * softplus(sum)), a head being `per_head` outputs
+    if (a_log) acc = expf(-expf(a_log[j / per_head]) * softplus_f(acc));
     z[(size_t)t * M + j] = acc;
 }
 
 extern "C" int vt_lowrank_tanh(const void* x, int x_dtype, long long ldx, const void* w2, int w_dtype, const float* bias,
-                               float* z, int n, int L, int M, int act, hipStream_t stream) {
+                               float* z, int n, int L, int M, int act, const float* a_log, int per_head,
+                               hipStream_t stream) {
     VT_REQUIRE(n >= 0 && L > 0 && L <= 8192 && M > 0 && ldx >= L, "vt_lowrank_tanh: bad sizes n=%d L=%d M=%d", n, L, M);
     VT_REQUIRE(act == 0 || act == 1, "vt_lowrank_tanh: act %d (0: none, 1: tanh)", act);
+    VT_REQUIRE(!a_log || (per_head > 0 && M % per_head == 0), "vt_lowrank_tanh: %d outputs in heads of %d", M, per_head);
     VT_REQUIRE(M <= 65535 * 256, "vt_lowrank_tanh: too many outputs");
     if (n == 0) return 0;
     const dim3 grid(n, (M + 255) / 256);
     const size_t lds = (size_t)L * sizeof(float);
     if (x_dtype == VT_F32 && w_dtype == VT_F32)
-        lowrank_tanh_kernel<float, float><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const float*)w2, bias, z, L, M, act);
+        lowrank_tanh_kernel<float, float><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const float*)w2, bias, z, L, M, act, a_log, per_head);
     else if (x_dtype == VT_F32 && w_dtype == VT_BF16)
-        lowrank_tanh_kernel<float, bf16_t><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const bf16_t*)w2, bias, z, L, M, act);
+        lowrank_tanh_kernel<float, bf16_t><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const bf16_t*)w2, bias, z, L, M, act, a_log, per_head);
     else if (x_dtype == VT_BF16 && w_dtype == VT_BF16)
-        lowrank_tanh_kernel<bf16_t, bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w2, bias, z, L, M, act);
+        lowrank_tanh_kernel<bf16_t, bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w2, bias, z, L, M, act, a_log, per_head);
     else return vt_fail("vt_lowrank_tanh: dtypes %d / %d are not handled", x_dtype, w_dtype);
     VT_CHECK_LAUNCH("vt_lowrank_tanh");
     return 0;
@@ -609,8 +615,7 @@ extern "C" int vt_general_delta(const void* x, int dtype, long long ldx, int r_c
 struct ChannelDeltaArgs {
     const void* qkv;        // [n][C]: q (G x D), k (G x D), v (H x Dv), after convolution and SiLU
     const void* beta;       // beta[t * ldb + h]: logits of the write strength
-    const float* z;         // [n][H * D] decay logits, float32
-    const float* a_log;     // [H]
+    const float* g;         // [n][H * D] decays, float32
     float* state;           // slot s: state + s * slot_stride, [H][Dv][D]
     const int* entry_start;
     const int* slots;
@@ -644,7 +649,6 @@ __global__ __launch_bounds__(256) void delta_rule_channel_kernel(ChannelDeltaArg
     const TI* x = (const TI*)a.qkv;
     const TB* bl = (const TB*)a.beta;
     const int col = col0 + cl;
-    const float decay_rate = expf(a.a_log[h]);
     const float q_scale = 1.0f / sqrtf((float)D);
 
     float S[DS];
@@ -666,7 +670,7 @@ __global__ __launch_bounds__(256) void delta_rule_channel_kernel(ChannelDeltaArg
             const bool in = ok && d < D;
             in_q[i] = in ? load_f32<TI>(x, row + (size_t)kh * D + d) : 0.f;
             in_k[i] = in ? load_f32<TI>(x, row + (size_t)(G + kh) * D + d) : 0.f;
-            in_z[i] = in ? a.z[zrow + d] : 0.f;
+            in_z[i] = in ? a.g[zrow + d] : 0.f;
         }
         const int j = col0 + r;
         in_v = (ok && j < Dv) ? load_f32<TI>(x, row + (size_t)2 * G * D + (size_t)h * Dv + j) : 0.f;
@@ -691,7 +695,7 @@ __global__ __launch_bounds__(256) void delta_rule_channel_kernel(ChannelDeltaArg
                 const int d = DS * r + i;
                 qs[cl][d] = in_q[i] * rq;
                 ks[cl][d] = in_k[i] * rk;
-                gs[cl][d] = expf(-decay_rate * softplus_f(in_z[i]));
+                gs[cl][d] = in_z[i];
             }
             vs[cl][r] = in_v;
             if (r == 0) beta_s[cl] = 1.0f / (1.0f + expf(-in_b));
@@ -733,7 +737,7 @@ __global__ __launch_bounds__(256) void delta_rule_channel_kernel(ChannelDeltaArg
 }
 
 extern "C" int vt_delta_rule_channel(const void* qkv, int dtype, const void* beta, int beta_dtype, long long ldb,
-                                     const float* z, const float* a_log, float* state, long long slot_stride,
+                                     const float* g, float* state, long long slot_stride,
                                      const int* entry_start, const int* slots, float* o, int n_entries, int H, int G, int D,
                                      int Dv, hipStream_t stream) {
     VT_REQUIRE(n_entries >= 0 && H > 0 && G > 0 && H % G == 0, "vt_delta_rule_channel: bad heads %d/%d", H, G);
@@ -743,7 +747,7 @@ extern "C" int vt_delta_rule_channel(const void* qkv, int dtype, const void* bet
     VT_REQUIRE(H <= 65535, "vt_delta_rule_channel: too many heads (%d)", H);
     if (n_entries == 0) return 0;
     ChannelDeltaArgs a;
-    a.qkv = qkv; a.beta = beta; a.z = z; a.a_log = a_log; a.state = state; a.entry_start = entry_start; a.slots = slots;
+    a.qkv = qkv; a.beta = beta; a.g = g; a.state = state; a.entry_start = entry_start; a.slots = slots;
     a.o = o; a.slot_stride = slot_stride; a.ldb = ldb; a.H = H; a.G = G; a.D = D; a.Dv = Dv;
     const int share = (D + 15) / 16;
     const dim3 grid(n_entries, H, (Dv + DELTA_GROUPS - 1) / DELTA_GROUPS);
@@ -789,7 +793,7 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(MemoryArgs a) {
     __shared__ __attribute__((aligned(16))) float qs[TILE][DP];
     __shared__ __attribute__((aligned(16))) float ks[TILE][DP];
     __shared__ float vs[TILE][DELTA_GROUPS];
-    __shared__ float i_s[TILE], f_s[TILE];
+    __shared__ float i_s[TILE], f_s[TILE], keep_s[TILE], put_s[TILE], floor_s[TILE];
 
     const int e = blockIdx.x, h = blockIdx.y, zb = blockIdx.z, col0 = zb * DELTA_GROUPS;
     const int ZB = gridDim.z;
@@ -854,11 +858,29 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(MemoryArgs a) {
         }
         __syncthreads();
         if (t0 + TILE < end) fetch(t0 + TILE);      // on its way while this tile is worked through
+        {
+            // The running maximum is a chain of additions and maxima, token by token, that every thread walks for
+            // itself (it is the same whatever the tile); the thread of token cl then works out that token's three
+            // exponentials, so that they leave the recurrence below: keep = e^(f + m - m'), put = e^(i - m'), and
+            // e^(-m'), the least that the normalizer's product counts as.
+            float lf_own = 0.f, li_own = 0.f, m_own_new = 0.f;
+#pragma unroll
+            for (int tt = 0; tt < TILE; ++tt) {
+                if (tt < nt) {
+                    const float lf = f_s[tt] + m, li = i_s[tt];
+                    m = fmaxf(lf, li);
+                    if (tt == cl) { lf_own = lf; li_own = li; m_own_new = m; }
+                }
+            }
+            if (cl < nt && r == 0) {
+                keep_s[cl] = expf(lf_own - m_own_new);
+                put_s[cl] = expf(li_own - m_own_new);
+                floor_s[cl] = expf(-m_own_new);
+            }
+        }
+        __syncthreads();
         auto token = [&](int tt) {
-            const float lf = f_s[tt] + m, li = i_s[tt];
-            const float m_new = fmaxf(lf, li);
-            const float keep = expf(lf - m_new), put = expf(li - m_new);
-            m = m_new;
+            const float keep = keep_s[tt], put = put_s[tt];
             const float pv = put * vs[tt][cl];
             float acc = 0.f, den = 0.f;
 #pragma unroll
@@ -873,7 +895,7 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(MemoryArgs a) {
             acc = row16_sum(acc);
             den = row16_sum(den);
             if (r == 0 && col < Dv)
-                a.o[((size_t)(t0 + tt) * H + h) * Dv + col] = acc / (fmaxf(fabsf(den), expf(-m_new)) + 1e-6f);
+                a.o[((size_t)(t0 + tt) * H + h) * Dv + col] = acc / (fmaxf(fabsf(den), floor_s[tt]) + 1e-6f);
         };
         if (nt == TILE) {
 #pragma unroll

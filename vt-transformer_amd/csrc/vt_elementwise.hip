@@ -185,10 +185,12 @@ extern "C" int vt_rmsnorm(float* h, const void* delta, int delta_dtype, const fl
 // Layer norm with gain and bias, fused with the residual additions in front of it:
 //     x = h[row] + (delta[row] + delta2[row]);   out = (x - mean) / sqrt(var + eps) * gain + bias
 // with var the mean of the squared deviations from the mean (two sums, the second over x - mean), all in float32.
-// A thread keeps its values in registers between the sums and the scaling (up to LN_MAXV * 256 columns; wider rows
-// are read again).  With `update` the sum x is written back to h.
+// A thread keeps its values in registers between the sums and the scaling (widths that are a multiple of 4, up to
+// LN_MAXV * 1024 columns; other rows are read again).  With `update` the sum x is written back to h.
 // ---------------------------------------------------------------------------
 #define LN_MAXV 16
+// NV > 0: widths that are a multiple of 4, every value read once with 16-byte loads (NV of them per thread) and kept in
+// registers; NV == 0: any width, the row is read again for the second sum and for the scaling.
 template <typename TD, typename TO, int NV>
 __global__ __launch_bounds__(256) void layernorm_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                                        const TD* __restrict__ delta2, const float* __restrict__ gain,
@@ -200,71 +202,90 @@ __global__ __launch_bounds__(256) void layernorm_kernel(float* __restrict__ h, c
     float* hr = h + src * hidden;
     const TD* d1 = delta ? delta + src * hidden : nullptr;
     const TD* d2 = delta2 ? delta2 + src * hidden : nullptr;
+    TO* o = out + (size_t)r * hidden;
+    if (NV > 0) {
+        const int nq = hidden >> 2;
+        float4 x[NV > 0 ? NV : 1];
+        float sum = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int qi = tid + v * 256;
+            x[v] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (qi < nq) {
+                x[v] = load4(hr + 4 * qi);
+                if (d1) {
+                    float4 a = load4(d1 + 4 * qi);
+                    if (d2) {
+                        const float4 b = load4(d2 + 4 * qi);
+                        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+                    }
+                    x[v].x += a.x; x[v].y += a.y; x[v].z += a.z; x[v].w += a.w;
+                    if (update) store4(hr + 4 * qi, x[v]);
+                }
+                sum += (x[v].x + x[v].y) + (x[v].z + x[v].w);
+            }
+        }
+        const float mean = block_sum(sum, red) / (float)hidden;
+        float sq = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int qi = tid + v * 256;
+            if (qi < nq) {
+                x[v].x -= mean; x[v].y -= mean; x[v].z -= mean; x[v].w -= mean;
+                sq += x[v].x * x[v].x + x[v].y * x[v].y + x[v].z * x[v].z + x[v].w * x[v].w;
+            }
+        }
+        const float rinv = 1.0f / sqrtf(block_sum(sq, red) / (float)hidden + eps);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int qi = tid + v * 256;
+            if (qi < nq) {
+                const float4 g = load4(gain + 4 * qi);
+                const float4 b = bias ? load4(bias + 4 * qi) : make_float4(0.f, 0.f, 0.f, 0.f);
+                store4(o + 4 * qi, make_float4(fmaf(x[v].x * rinv, g.x, b.x), fmaf(x[v].y * rinv, g.y, b.y),
+                                               fmaf(x[v].z * rinv, g.z, b.z), fmaf(x[v].w * rinv, g.w, b.w)));
+            }
+        }
+        return;
+    }
     auto value = [&](int i) -> float {
         float x = hr[i];
         if (d1 && d2) x += load_f32<TD>(d1, i) + load_f32<TD>(d2, i);
         else if (d1) x += load_f32<TD>(d1, i);
         return x;
     };
-    float x[NV > 0 ? NV : 1];
     float sum = 0.f;
-    if (NV > 0) {
-#pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const int i = tid + v * 256;
-            x[v] = i < hidden ? value(i) : 0.f;
-            if (i < hidden && update && d1) hr[i] = x[v];
-            sum += x[v];
-        }
-    } else {
-        for (int i = tid; i < hidden; i += 256) {
-            const float xv = value(i);
-            if (update && d1) hr[i] = xv;
-            sum += xv;
-        }
-        __syncthreads();
-        d1 = update && d1 ? nullptr : d1;       // (h now holds the sum)
-        if (!d1) d2 = nullptr;
+    for (int i = tid; i < hidden; i += 256) {
+        const float xv = value(i);
+        if (update && d1) hr[i] = xv;
+        sum += xv;
     }
+    __syncthreads();
+    if (update && d1) d1 = d2 = nullptr;        // (h now holds the sum)
     const float mean = block_sum(sum, red) / (float)hidden;
     float sq = 0.f;
-    if (NV > 0) {
-#pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const int i = tid + v * 256;
-            const float dv = i < hidden ? x[v] - mean : 0.f;
-            sq = fmaf(dv, dv, sq);
-        }
-    } else {
-        for (int i = tid; i < hidden; i += 256) {
-            const float dv = value(i) - mean;
-            sq = fmaf(dv, dv, sq);
-        }
+    for (int i = tid; i < hidden; i += 256) {
+        const float dv = value(i) - mean;
+        sq = fmaf(dv, dv, sq);
     }
     const float rinv = 1.0f / sqrtf(block_sum(sq, red) / (float)hidden + eps);
-    TO* o = out + (size_t)r * hidden;
-    if (NV > 0) {
-#pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const int i = tid + v * 256;
-            if (i < hidden) store_f32<TO>(o, i, fmaf((x[v] - mean) * rinv, gain[i], bias ? bias[i] : 0.f));
-        }
-    } else {
-        for (int i = tid; i < hidden; i += 256)
-            store_f32<TO>(o, i, fmaf((value(i) - mean) * rinv, gain[i], bias ? bias[i] : 0.f));
-    }
+    for (int i = tid; i < hidden; i += 256)
+        store_f32<TO>(o, i, fmaf((value(i) - mean) * rinv, gain[i], bias ? bias[i] : 0.f));
 }
 
 template <typename TD, typename TO>
 static void launch_layernorm(float* h, const void* delta, const void* delta2, const float* gain, const float* bias, void* out,
                              const int* rows, int n_out, int hidden, float eps, int update_h, hipStream_t stream) {
+    const bool aligned = (hidden % 4 == 0) && !((uintptr_t)h & 15) && !((uintptr_t)gain & 15) && !((uintptr_t)bias & 15) &&
+                         !((uintptr_t)out & 15) && !((uintptr_t)delta & 15) && !((uintptr_t)delta2 & 15);
+    const int nq = hidden / 4;
 #define VT_LN(NV) layernorm_kernel<TD, TO, NV><<<n_out, 256, 0, stream>>>(h, (const TD*)delta, (const TD*)delta2, gain, bias, \
                                                                          (TO*)out, rows, hidden, eps, update_h)
-    if (hidden <= 256) VT_LN(1);
-    else if (hidden <= 512) VT_LN(2);
-    else if (hidden <= 1024) VT_LN(4);
-    else if (hidden <= 2048) VT_LN(8);
-    else if (hidden <= 256 * LN_MAXV) VT_LN(LN_MAXV);
+    if (aligned && nq <= 256 * 1) VT_LN(1);
+    else if (aligned && nq <= 256 * 2) VT_LN(2);
+    else if (aligned && nq <= 256 * 4) VT_LN(4);
+    else if (aligned && nq <= 256 * 8) VT_LN(8);
+    else if (aligned && nq <= 256 * LN_MAXV) VT_LN(LN_MAXV);
     else VT_LN(0);
 #undef VT_LN
 }

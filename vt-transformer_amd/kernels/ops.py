@@ -1239,10 +1239,11 @@ def gated_rmsnorm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, gat
 
 
 def lowrank_tanh(x: torch.Tensor, x_column: int, w2: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-                 tanh: bool = True) -> torch.Tensor:
+                 tanh: bool = True, decay: Optional[tuple] = None) -> torch.Tensor:
     """out[t, j] = bias[j] + sum_l w2[j, l] * tanh(x[t, x_column + l]): float32 sums in the order of l, float32 results.
     x: a 2-d tensor whose rows are the tokens'; w2 [M, L] in float32 or the 16-bit type.  tanh False: the low-rank part
-    enters as it is (the second half of a linear low-rank projection, kept in float32)."""
+    enters as it is (the second half of a linear low-rank projection, kept in float32).  decay (a_log, per_head): the
+    sums leave as decays, out = exp(-exp(a_log[j // per_head]) * softplus(sum)), a_log float32 [M / per_head]."""
     n = x.shape[0]
     m, low = w2.shape
     _chk(x, "lowrank_tanh.x")
@@ -1254,9 +1255,15 @@ def lowrank_tanh(x: torch.Tensor, x_column: int, w2: torch.Tensor, bias: Optiona
     if bias is not None:
         _chk(bias, "lowrank_tanh.bias", torch.float32, (m,))
     _chk(out, "lowrank_tanh.out", torch.float32, (n, m))
+    a_log, per_head = decay if decay is not None else (None, 0)
+    if a_log is not None:
+        if per_head <= 0 or m % per_head:
+            raise KernelError(f"lowrank_tanh: {m} outputs in heads of {per_head}")
+        _chk(a_log, "lowrank_tanh.a_log", torch.float32, (m // per_head,))
     xptr = ctypes.c_void_p(x.data_ptr() + x_column * x.element_size())
     _run(load_lib("vt_delta", half=_half(x, w2)), "vt_lowrank_tanh", xptr, _i(_code(x)), ctypes.c_longlong(x.stride(0)),
-         _ptr(w2), _i(_code(w2)), _ptr(bias), _ptr(out), _i(n), _i(low), _i(m), _i(1 if tanh else 0), _stream())
+         _ptr(w2), _i(_code(w2)), _ptr(bias), _ptr(out), _i(n), _i(low), _i(m), _i(1 if tanh else 0), _ptr(a_log),
+         _i(per_head), _stream())
     return out
 
 
@@ -1290,13 +1297,13 @@ def general_delta(x: torch.Tensor, r_column: int, k_column: int, v_column: int, 
     return out
 
 
-def delta_rule_channel(qkv: torch.Tensor, beta: torch.Tensor, beta_column: int, decay_logits: torch.Tensor,
-                       a_log: torch.Tensor, state: torch.Tensor, entry_start: torch.Tensor, slots: torch.Tensor,
+def delta_rule_channel(qkv: torch.Tensor, beta: torch.Tensor, beta_column: int, decays: torch.Tensor,
+                       state: torch.Tensor, entry_start: torch.Tensor, slots: torch.Tensor,
                        out: torch.Tensor, n_heads: int, n_kv: int, key_dim: int, value_dim: int) -> torch.Tensor:
-    """The gated delta rule with a decay per key channel, S <- diag(g) S with g = exp(-exp(a_log[h]) softplus(z)), over
-    the tokens of every entry, from and into state[slot] ([H, Dv, D] float32).  qkv as for delta_rule; beta: a 2-d
-    tensor whose rows are the tokens', with the H logits of the write strength from column beta_column; decay_logits
-    z [n, H * D] float32; out [n, H * Dv] float32."""
+    """The gated delta rule with a decay per key channel, S <- diag(g) S, over the tokens of every entry, from and
+    into state[slot] ([H, Dv, D] float32).  qkv as for delta_rule; beta: a 2-d tensor whose rows are the tokens', with
+    the H logits of the write strength from column beta_column; decays g [n, H * D] float32 (lowrank_tanh with
+    `decay` makes them); out [n, H * Dv] float32."""
     n = qkv.shape[0]
     c = 2 * n_kv * key_dim + n_heads * value_dim
     _chk(qkv, "delta_rule_channel.qkv", None, (n, c))
@@ -1305,8 +1312,7 @@ def delta_rule_channel(qkv: torch.Tensor, beta: torch.Tensor, beta_column: int, 
         raise KernelError(f"delta_rule_channel.beta: shape {tuple(beta.shape)} has no {n_heads} columns from {beta_column}")
     if beta.dtype != torch.float32 and beta.dtype != qkv.dtype:
         raise KernelError(f"delta_rule_channel: logits of dtype {beta.dtype} beside inputs of {qkv.dtype}")
-    _chk(decay_logits, "delta_rule_channel.decay_logits", torch.float32, (n, n_heads * key_dim))
-    _chk(a_log, "delta_rule_channel.a_log", torch.float32, (n_heads,))
+    _chk(decays, "delta_rule_channel.decays", torch.float32, (n, n_heads * key_dim))
     _chk(out, "delta_rule_channel.out", torch.float32, (n, n_heads * value_dim))
     _chk(entry_start, "delta_rule_channel.entry_start", torch.int32)
     _chk(slots, "delta_rule_channel.slots", torch.int32)
@@ -1315,7 +1321,7 @@ def delta_rule_channel(qkv: torch.Tensor, beta: torch.Tensor, beta_column: int, 
     sp, ss = _state_rows(state, "delta_rule_channel", n_heads * key_dim * value_dim)
     bptr = ctypes.c_void_p(beta.data_ptr() + beta_column * beta.element_size())
     _run(load_lib("vt_delta", half=_half(qkv, beta)), "vt_delta_rule_channel", _ptr(qkv), _i(_code(qkv)), bptr, _i(_code(beta)),
-         ctypes.c_longlong(beta.stride(0)), _ptr(decay_logits), _ptr(a_log), sp, ss, _ptr(entry_start), _ptr(slots),
+         ctypes.c_longlong(beta.stride(0)), _ptr(decays), sp, ss, _ptr(entry_start), _ptr(slots),
          _ptr(out), _i(entry_start.numel() - 1), _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _stream())
     return out
 

@@ -157,9 +157,11 @@ class GatedDeltaMixer(Part):
             ops.short_conv_carry(y, c, self.taps, conv_state, ctx.entry_start, ctx.state_slots)
         o = rt.buffer("delta.o", (n, self.nh * self.dv), torch.float32)
         if self.channel_decay:
-            logits = ops.lowrank_tanh(y, self.col_decay, self.w_a2, self.dt_bias,
-                                      rt.buffer("delta.decay", (n, self.nh * self.d), torch.float32), tanh=False)
-            ops.delta_rule_channel(qkv, y, self.col_beta, logits, self.a_log, rule_state, ctx.entry_start, ctx.state_slots, o,
+            # (the decays of all tokens at once, so that the recurrence only multiplies by them)
+            decays = ops.lowrank_tanh(y, self.col_decay, self.w_a2, self.dt_bias,
+                                      rt.buffer("delta.decay", (n, self.nh * self.d), torch.float32), tanh=False,
+                                      decay=(self.a_log, self.d))
+            ops.delta_rule_channel(qkv, y, self.col_beta, decays, rule_state, ctx.entry_start, ctx.state_slots, o,
                                    self.nh, self.nkv, self.d, self.dv)
         else:
             ops.delta_rule(qkv, y, self.col_beta, self.a_log, self.dt_bias, rule_state, ctx.entry_start, ctx.state_slots, o,

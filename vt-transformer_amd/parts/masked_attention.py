@@ -243,7 +243,8 @@ class MaskedAttention(Part):
             t[nm["k_norm"]] = TensorDecl((self.d,), "gain")
         if self.distance_log:
             t[nm["r1"]] = TensorDecl((self.nh,), "bias")
-            t[nm["r2"]] = TensorDecl((self.nh,), "bias")
+            # (r2 multiplies the distance inside the logarithm: a model with random weights draws it around 1)
+            t[nm["r2"]] = TensorDecl((self.nh,), "gain")
         if self.score_shift:
             t[nm["shift"]] = TensorDecl((self.nh,), "bias")
         if self.o_bias:
@@ -282,7 +283,7 @@ class MaskedAttention(Part):
         if self.qk_gain:
             self.q_gain, self.k_gain = rt.place(get(nm["q_norm"]), "gain"), rt.place(get(nm["k_norm"]), "gain")
         if self.distance_log:
-            self.r1, self.r2 = rt.place(get(nm["r1"]), "bias"), rt.place(get(nm["r2"]), "bias")
+            self.r1, self.r2 = rt.place(get(nm["r1"]), "bias"), rt.place(get(nm["r2"]), "gain")
         if self.score_shift:
             self.shift = rt.place(get(nm["shift"]), "bias")
         if self.o_bias:
