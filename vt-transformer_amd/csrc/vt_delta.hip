@@ -410,24 +410,39 @@ extern "C" int vt_gated_rmsnorm(const float* o, const float* w, const void* gate
 
 // ---------------------------------------------------------------------------
 // z[t][j] = bias[j] + sum_l W2[j][l] * tanh(x[t * ldx + l]), l = 0, 1, .. in that order, float32
-template <typename TI, typename TW>
+// A block takes TB tokens and 256 outputs: a thread reads its row of W2 once for all of them (the rows of neighbouring
+// threads lie L elements apart, so each read of W2 touches as many cache lines as the wave has lanes: with many tokens
+// it is what the kernel waits for, and TB tokens share it).  The sums add up in the order of l whatever TB.
+template <typename TI, typename TW, int TB>
 __global__ __launch_bounds__(256) void lowrank_tanh_kernel(const TI* __restrict__ x, long long ldx, const TW* __restrict__ w2,
-                                                           const float* __restrict__ bias, float* __restrict__ z, int L, int M,
-                                                           int act, const float* __restrict__ a_log, int per_head) {
-    extern __shared__ float th[];
-    const int t = blockIdx.x;
-    for (int l = threadIdx.x; l < L; l += 256) {
-        const float v = load_f32<TI>(x, (size_t)t * ldx + l);
-        th[l] = act ? tanhf(v) : v;
+                                                           const float* __restrict__ bias, float* __restrict__ z, int n, int L,
+                                                           int M, int act, const float* __restrict__ a_log, int per_head) {
+    extern __shared__ float th[];       // [TB][L]
+    const int t0 = blockIdx.x * TB;
+    for (int i = threadIdx.x; i < TB * L; i += 256) {
+        const int tb = i / L, l = i - tb * L;
+        const float v = t0 + tb < n ? load_f32<TI>(x, (size_t)(t0 + tb) * ldx + l) : 0.f;
+        th[i] = act ? tanhf(v) : v;
     }
     __syncthreads();
     const int j = blockIdx.y * 256 + threadIdx.x;
     if (j >= M) return;
-    float acc = bias ? bias[j] : 0.f;
-    for (int l = 0; l < L; ++l) acc = fmaf(load_f32<TW>(w2, (size_t)j * L + l), th[l], acc);
+    float acc[TB];
+    const float b0 = bias ? bias[j] : 0.f;
+#pragma unroll
+    for (int tb = 0; tb < TB; ++tb) acc[tb] = b0;
+    for (int l = 0; l < L; ++l) {
+        const float w = load_f32<TW>(w2, (size_t)j * L + l);
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb) acc[tb] = fmaf(w, th[tb * L + l], acc[tb]);
+    }
     // the sums as decay logits: out = exp(-exp(a_log[head]) * softplus(sum)), a head being `per_head` outputs
-    if (a_log) acc = expf(-expf(a_log[j / per_head]) * softplus_f(acc));
-    z[(size_t)t * M + j] = acc;
+    const float rate = a_log ? expf(a_log[j / per_head]) : 0.f;
+#pragma unroll
+    for (int tb = 0; tb < TB; ++tb) {
+        if (t0 + tb >= n) break;
+        z[(size_t)(t0 + tb) * M + j] = a_log ? expf(-rate * softplus_f(acc[tb])) : acc[tb];
+    }
 }
 
 extern "C" int vt_lowrank_tanh(const void* x, int x_dtype, long long ldx, const void* w2, int w_dtype, const float* bias,
@@ -438,15 +453,21 @@ extern "C" int vt_lowrank_tanh(const void* x, int x_dtype, long long ldx, const 
     VT_REQUIRE(!a_log || (per_head > 0 && M % per_head == 0), "vt_lowrank_tanh: %d outputs in heads of %d", M, per_head);
     VT_REQUIRE(M <= 65535 * 256, "vt_lowrank_tanh: too many outputs");
     if (n == 0) return 0;
-    const dim3 grid(n, (M + 255) / 256);
-    const size_t lds = (size_t)L * sizeof(float);
-    if (x_dtype == VT_F32 && w_dtype == VT_F32)
-        lowrank_tanh_kernel<float, float><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const float*)w2, bias, z, L, M, act, a_log, per_head);
-    else if (x_dtype == VT_F32 && w_dtype == VT_BF16)
-        lowrank_tanh_kernel<float, bf16_t><<<grid, 256, lds, stream>>>((const float*)x, ldx, (const bf16_t*)w2, bias, z, L, M, act, a_log, per_head);
-    else if (x_dtype == VT_BF16 && w_dtype == VT_BF16)
-        lowrank_tanh_kernel<bf16_t, bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w2, bias, z, L, M, act, a_log, per_head);
+    // many tokens and a short middle: eight tokens to a block
+    const bool many = n >= 256 && L <= 1024;
+    const int tb = many ? 8 : 1;
+    const dim3 grid((n + tb - 1) / tb, (M + 255) / 256);
+    const size_t lds = (size_t)tb * L * sizeof(float);
+#define VT_LOWRANK(TI, TW)                                                                                                  \
+    do {                                                                                                                    \
+        if (many) lowrank_tanh_kernel<TI, TW, 8><<<grid, 256, lds, stream>>>((const TI*)x, ldx, (const TW*)w2, bias, z, n, L, M, act, a_log, per_head); \
+        else lowrank_tanh_kernel<TI, TW, 1><<<grid, 256, lds, stream>>>((const TI*)x, ldx, (const TW*)w2, bias, z, n, L, M, act, a_log, per_head);      \
+    } while (0)
+    if (x_dtype == VT_F32 && w_dtype == VT_F32) VT_LOWRANK(float, float);
+    else if (x_dtype == VT_F32 && w_dtype == VT_BF16) VT_LOWRANK(float, bf16_t);
+    else if (x_dtype == VT_BF16 && w_dtype == VT_BF16) VT_LOWRANK(bf16_t, bf16_t);
     else return vt_fail("vt_lowrank_tanh: dtypes %d / %d are not handled", x_dtype, w_dtype);
+#undef VT_LOWRANK
     VT_CHECK_LAUNCH("vt_lowrank_tanh");
     return 0;
 }
@@ -612,6 +633,14 @@ extern "C" int vt_general_delta(const void* x, int dtype, long long ldx, int r_c
 }
 
 // ---------------------------------------------------------------------------
+// Which state element lane r (of a row of 16) holds as its i-th: groups of four consecutive elements, the groups dealt
+// out to the lanes in turn (element 4 (r + 16 j) + e for i = 4 j + e), so that a row of lanes reads 256 consecutive bytes
+// of the state or of a token's vectors with every 16-byte access; heads of up to 32 elements: DS consecutive ones.
+template <int DS>
+__device__ __forceinline__ constexpr int lane_elem(int r, int i) {
+    return DS <= 4 ? DS * r + i : 4 * (r + 16 * (i / 4)) + (i % 4);
+}
+
 struct ChannelDeltaArgs {
     const void* qkv;        // [n][C]: q (G x D), k (G x D), v (H x Dv), after convolution and SiLU
     const void* beta;       // beta[t * ldb + h]: logits of the write strength
@@ -624,8 +653,8 @@ struct ChannelDeltaArgs {
     int H, G, D, Dv;
 };
 
-// vt_general_delta's arrangement: 16 rows of lanes for the recurrence (a row per value column, lane r holding the DS
-// consecutive state elements from d = DS r) and TILE tokens x 16 lanes for a tile's inputs.  Per token and column, with
+// vt_general_delta's arrangement: 16 rows of lanes for the recurrence (a row per value column, lane r holding DS state
+// elements in groups of four: lane_elem) and TILE tokens x 16 lanes for a tile's inputs.  Per token and column, with
 // k' and q' the unit vectors (q' also times D^-1/2):
 //     S_d <- g_d S_d;  p = k' . S;  u = beta (v - p);  S_d <- S_d + k'_d u;  o = q' . S
 // the same instructions in the same order whatever the tile, so nothing depends on how a request was cut.
@@ -654,7 +683,7 @@ __global__ __launch_bounds__(256) void delta_rule_channel_kernel(ChannelDeltaArg
     float S[DS];
 #pragma unroll
     for (int i = 0; i < DS; ++i) {
-        const int d = DS * r + i;
+        const int d = lane_elem<DS>(r, i);
         S[i] = (col < Dv && d < D) ? S_head[(size_t)col * D + d] : 0.f;
     }
 
@@ -666,7 +695,7 @@ __global__ __launch_bounds__(256) void delta_rule_channel_kernel(ChannelDeltaArg
         const size_t zrow = (size_t)(ok ? t : start) * H * D + (size_t)h * D;
 #pragma unroll
         for (int i = 0; i < DS; ++i) {
-            const int d = DS * r + i;
+            const int d = lane_elem<DS>(r, i);
             const bool in = ok && d < D;
             in_q[i] = in ? load_f32<TI>(x, row + (size_t)kh * D + d) : 0.f;
             in_k[i] = in ? load_f32<TI>(x, row + (size_t)(G + kh) * D + d) : 0.f;
@@ -692,7 +721,7 @@ __global__ __launch_bounds__(256) void delta_rule_channel_kernel(ChannelDeltaArg
             const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
 #pragma unroll
             for (int i = 0; i < DS; ++i) {
-                const int d = DS * r + i;
+                const int d = lane_elem<DS>(r, i);
                 qs[cl][d] = in_q[i] * rq;
                 ks[cl][d] = in_k[i] * rk;
                 gs[cl][d] = in_z[i];
@@ -706,7 +735,7 @@ __global__ __launch_bounds__(256) void delta_rule_channel_kernel(ChannelDeltaArg
             float p = 0.f;
 #pragma unroll
             for (int i = 0; i < DS; ++i) {
-                const int d = DS * r + i;
+                const int d = lane_elem<DS>(r, i);
                 S[i] *= gs[tt][d];
                 p = fmaf(ks[tt][d], S[i], p);
             }
@@ -715,7 +744,7 @@ __global__ __launch_bounds__(256) void delta_rule_channel_kernel(ChannelDeltaArg
             float acc = 0.f;
 #pragma unroll
             for (int i = 0; i < DS; ++i) {
-                const int d = DS * r + i;
+                const int d = lane_elem<DS>(r, i);
                 S[i] = fmaf(ks[tt][d], u, S[i]);
                 acc = fmaf(qs[tt][d], S[i], acc);
             }
@@ -731,7 +760,7 @@ __global__ __launch_bounds__(256) void delta_rule_channel_kernel(ChannelDeltaArg
     }
 #pragma unroll
     for (int i = 0; i < DS; ++i) {
-        const int d = DS * r + i;
+        const int d = lane_elem<DS>(r, i);
         if (col < Dv && d < D) S_head[(size_t)col * D + d] = S[i];
     }
 }
@@ -812,7 +841,7 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(MemoryArgs a) {
     float S[DS], nn[DS];
 #pragma unroll
     for (int i = 0; i < DS; ++i) {
-        const int d = DS * r + i;
+        const int d = lane_elem<DS>(r, i);
         S[i] = (col < Dv && d < D) ? S_head[(size_t)col * D + d] : 0.f;
         nn[i] = d < D ? n_own[d] : 0.f;
     }
@@ -825,7 +854,7 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(MemoryArgs a) {
         const size_t row = (size_t)(ok ? t : start) * a.ldx;
 #pragma unroll
         for (int i = 0; i < DS; ++i) {
-            const int d = DS * r + i;
+            const int d = lane_elem<DS>(r, i);
             const bool in = ok && d < D;
             in_q[i] = in ? load_f32<TI>(x, row + a.q_col + (size_t)h * D + d) : 0.f;
             in_k[i] = in ? load_f32<TI>(x, row + a.k_col + (size_t)h * D + d) : 0.f;
@@ -844,7 +873,7 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(MemoryArgs a) {
         if (cl < TILE) {
 #pragma unroll
             for (int i = 0; i < DS; ++i) {
-                const int d = DS * r + i;
+                const int d = lane_elem<DS>(r, i);
                 qs[cl][d] = in_q[i] * a.q_scale;
                 ks[cl][d] = in_k[i];
             }
@@ -885,7 +914,7 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(MemoryArgs a) {
             float acc = 0.f, den = 0.f;
 #pragma unroll
             for (int i = 0; i < DS; ++i) {
-                const int d = DS * r + i;
+                const int d = lane_elem<DS>(r, i);
                 const float kd = ks[tt][d], qd = qs[tt][d];
                 S[i] = fmaf(keep, S[i], kd * pv);
                 nn[i] = fmaf(keep, nn[i], kd * put);
@@ -906,7 +935,7 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(MemoryArgs a) {
     }
 #pragma unroll
     for (int i = 0; i < DS; ++i) {
-        const int d = DS * r + i;
+        const int d = lane_elem<DS>(r, i);
         if (col < Dv && d < D) S_head[(size_t)col * D + d] = S[i];
         if (cl == 0 && d < D) n_own[d] = nn[i];
     }
