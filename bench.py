@@ -247,7 +247,7 @@ def fedovik_pair_configs(key: str, window: int):
                       "right": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "conv": 4,
                                 "a_rank": 64, "g_rank": 64},
                       "left_scale": 1.0, "right_scale": 1.0}}
-    mem = {"type": "mlstm", "mlp": mlp, "mixer": {"heads": heads, "dim": d, "vdim": d, "gate_cap": 15.0}}
+    mem = {"type": "mlstm", "mlp": mlp, "mixer": {"heads": heads, "dim": d, "vdim": d, "gate_cap": 12.0}}
     fed = {"architecture": "Fedovik", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6},
            "layers": [(att, pair, mem)[i % 3] for i in range(layers)], "loop": None, "max_positions": 32768}
     lis, _ = pair_configs(key, window)

@@ -212,3 +212,30 @@ def test_whole_model_prefix_property_and_layers():
         changed[name] = w[name] + 0.25 * torch.linspace(-1.0, 1.0, w[name].numel()).reshape(w[name].shape)
         assert float((pf.forward(cfg, changed, ids) - full).abs().max()) > 1e-4, name
     assert pf.greedy(cfg, w, ids[:5], 3) == pf.greedy(cfg, w, ids[:5], 3)
+
+
+def test_random_model_from_the_command_line(tmp_path):
+    """`--write-random-model` on a Fedovik config.json that says its low-rank sizes: every declared tensor is written,
+    the folder loads back into the same configuration, and the distance factor r2 is drawn around 1 (positive, as the
+    logarithm wants it)."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from vt_transformer_amd.config import load_config
+    from vt_transformer_amd.weights import WeightStore
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg_path = tmp_path / "c.json"
+    cfg_path.write_text(json.dumps(CONFIGS["C"]))
+    out = tmp_path / "m"
+    r = subprocess.run([sys.executable, "-m", "vt_transformer_amd", "--write-random-model", str(out), "--config", str(cfg_path),
+                        "--seed", "4"], capture_output=True, text=True, env=dict(os.environ, PYTHONPATH=root), timeout=300)
+    assert r.returncode == 0, r.stderr
+    cfg = load_config(str(out))
+    assert cfg.to_dict() == config_from_dict(copy.deepcopy(CONFIGS["C"])).to_dict()
+    store = WeightStore(str(out))
+    want = {k for k, d in declared_tensors(cfg).items() if not d.optional}
+    assert set(store.names()) == want
+    _, w = pf.read_folder(str(out))
+    assert float(w["l1.mix.left.r2"].min()) > 0.5
+    assert torch.isfinite(pf.forward(cfg.to_dict(), w, [3, 1, 4, 1, 5, 9, 2, 6])).all()
