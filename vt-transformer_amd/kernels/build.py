@@ -39,7 +39,8 @@ HALF_LIBS = ("vt_elementwise", "vt_gemm_bf16", "vt_attn_bf16", "vt_attn_masked",
              "vt_streams", "vt_moe")
 # the matrix-core kernel of the masked attention is built per (key size, value size) of a head
 DEFAULT_MASKED_DIMS = [(64, 64), (128, 128), (64, 96), (48, 80), (32, 48), (16, 16), (64, 32), (64, 16), (48, 32), (256, 192),
-                       (32, 16), (48, 48), (80, 48), (80, 64), (144, 128), (112, 48), (176, 48)]
+                       (32, 16), (48, 48), (80, 48), (80, 64), (144, 128), (112, 48), (176, 48), (16, 32), (16, 48), (16, 80),
+                       (16, 144), (64, 80)]
 
 
 class KernelBuildError(RuntimeError):
